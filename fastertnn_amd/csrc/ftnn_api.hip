@@ -1,0 +1,312 @@
+// C ABI of libftnn_hip.so: argument checking, the device-memory entry points, and
+// the reference's host-memory entry points built on top of them.
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "../../include/ftnn.h"
+#include "ftnn_internal.h"
+
+namespace ftnn {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+static int hip_fail(hipError_t e, const char* what) {
+    return fail(FTNN_EHIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// common conv-shape validation; fills OH/OW
+static int check_conv_shape(int N, int C, int H, int W, int H_pad, int W_pad, int kH, int kW,
+                            int H_stride, int W_stride, int* OH, int* OW) {
+    if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || kH <= 0 || kW <= 0 || H_stride <= 0 ||
+        W_stride <= 0 || H_pad < 0 || W_pad < 0)
+        return fail(FTNN_EINVAL, "non-positive dimension or negative padding");
+    if (H + 2 * H_pad < kH || W + 2 * W_pad < kW)
+        return fail(FTNN_EINVAL, "kernel %dx%d larger than padded input %dx%d", kH, kW,
+                    H + 2 * H_pad, W + 2 * W_pad);
+    if (N > 65535) return fail(FTNN_EINVAL, "batch %d above the supported 65535", N);
+    *OH = out_dim(H, H_pad, kH, H_stride);
+    *OW = out_dim(W, W_pad, kW, W_stride);
+    return FTNN_OK;
+}
+
+// ---- lazily created state behind the host-memory entry points ----
+struct HostCtx {
+    hipStream_t stream = nullptr;
+    void* buf[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    size_t cap[6] = {0, 0, 0, 0, 0, 0};
+};
+static HostCtx g_ctx;
+
+[[noreturn]] static void die(const char* what) {
+    // the reference reports failure by abort() (src/timing_layers.c:156-159)
+    fprintf(stderr, "libftnn_hip: %s: %s\n", what, g_err);
+    abort();
+}
+
+static void hip_or_die(hipError_t e, const char* what) {
+    if (e != hipSuccess) {
+        hip_fail(e, what);
+        die("HIP failure");
+    }
+}
+
+static hipStream_t host_stream() {
+    if (!g_ctx.stream) hip_or_die(hipStreamCreate(&g_ctx.stream), "hipStreamCreate");
+    return g_ctx.stream;
+}
+
+// grow-only device buffer number `slot`
+static void* dev_buf(int slot, size_t bytes) {
+    if (bytes == 0) bytes = 16;
+    if (g_ctx.cap[slot] < bytes) {
+        if (g_ctx.buf[slot]) {
+            hip_or_die(hipStreamSynchronize(host_stream()), "hipStreamSynchronize");
+            hip_or_die(hipFree(g_ctx.buf[slot]), "hipFree");
+        }
+        g_ctx.buf[slot] = nullptr;
+        g_ctx.cap[slot] = 0;
+        hip_or_die(hipMalloc(&g_ctx.buf[slot], bytes), "hipMalloc");
+        g_ctx.cap[slot] = bytes;
+    }
+    return g_ctx.buf[slot];
+}
+
+static void* upload(int slot, const void* host, size_t bytes) {
+    void* d = dev_buf(slot, bytes);
+    hip_or_die(hipMemcpyAsync(d, host, bytes, hipMemcpyHostToDevice, host_stream()), "H2D copy");
+    return d;
+}
+
+static void download(void* host, const void* dev, size_t bytes) {
+    hip_or_die(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, host_stream()), "D2H copy");
+    hip_or_die(hipStreamSynchronize(host_stream()), "hipStreamSynchronize");
+}
+
+static void* host_alloc(size_t bytes, bool aligned32) {
+    void* p;
+    if (aligned32) {
+        // aligned_alloc(32, ...) as src/tnns/ternarize2row_avx2.c:735
+        p = aligned_alloc(32, (bytes + 31) / 32 * 32);
+    } else {
+        p = malloc(bytes ? bytes : 1);
+    }
+    if (!p) {
+        fail(FTNN_ENOMEM, "host allocation of %zu bytes failed", bytes);
+        die("out of memory");
+    }
+    return p;
+}
+
+enum { SLOT_X = 0, SLOT_THR, SLOT_W, SLOT_ROWS, SLOT_SCRATCH, SLOT_Y };
+
+static int64_t* host_quantize_im2row(bool ternary, float* x, float* thr, int N, int C, int H, int W,
+                                     int H_pad, int W_pad, int kH, int kW, int H_stride,
+                                     int W_stride) {
+    int OH, OW;
+    if (check_conv_shape(N, C, H, W, H_pad, W_pad, kH, kW, H_stride, W_stride, &OH, &OW) != FTNN_OK)
+        die(ternary ? "t2r_p2_opt" : "b2r");
+    const size_t out_bytes =
+        (size_t)N * OH * OW * (size_t)ftnn_row_words(C, kH, kW, ternary) * sizeof(int64_t);
+    float* d_x = (float*)upload(SLOT_X, x, (size_t)N * C * H * W * sizeof(float));
+    float* d_thr = (float*)upload(SLOT_THR, thr, (size_t)N * sizeof(float));
+    int64_t* d_rows = (int64_t*)dev_buf(SLOT_ROWS, out_bytes);
+    void* d_scr = dev_buf(SLOT_SCRATCH, (size_t)ftnn_pack_scratch_bytes(N, C, H, W, ternary));
+    if (ftnn_quantize_im2row(ternary, d_x, d_thr, N, C, H, W, H_pad, W_pad, kH, kW, H_stride,
+                             W_stride, d_rows, d_scr, host_stream()) != FTNN_OK)
+        die(ternary ? "t2r_p2_opt" : "b2r");
+    int64_t* out = (int64_t*)host_alloc(out_bytes, true);
+    download(out, d_rows, out_bytes);
+    return out;
+}
+
+static float* host_mm(int type, int64_t* a, int64_t* b, int N, int OH, int OW, int KN, int K,
+                      int K_unpack, float alpha) {
+    if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0) {
+        fail(FTNN_EINVAL, "non-positive GEMM dimension");
+        die("mm");
+    }
+    const size_t M = (size_t)N * OH * OW;
+    const size_t kw = (size_t)round4(K);
+    const size_t a_words = kw * ((type == kTNN || type == kTBN) ? 2 : 1);
+    const size_t b_words = kw * ((type == kTNN || type == kBTN) ? 2 : 1);
+    int64_t* d_a = (int64_t*)upload(SLOT_ROWS, a, M * a_words * sizeof(int64_t));
+    int64_t* d_b = (int64_t*)upload(SLOT_W, b, (size_t)KN * b_words * sizeof(int64_t));
+    const size_t y_bytes = M * KN * sizeof(float);
+    float* d_y = (float*)dev_buf(SLOT_Y, y_bytes);
+    if (ftnn_mm(type, d_a, d_b, N, OH, OW, KN, K, K_unpack, alpha, d_y, host_stream()) != FTNN_OK)
+        die("mm");
+    float* y = (float*)host_alloc(y_bytes, false);
+    download(y, d_y, y_bytes);
+    return y;
+}
+
+}  // namespace ftnn
+
+using namespace ftnn;
+
+extern "C" {
+
+const char* ftnn_last_error(void) { return g_err; }
+
+const char* ftnn_version(void) { return "ftnn-hip 0.1 gfx950"; }
+
+int ftnn_out_dim(int in, int pad, int k, int stride) { return out_dim(in, pad, k, stride); }
+
+int64_t ftnn_row_words(int C, int KH, int KW, int ternary) {
+    const int64_t kw = round4(cpack_of(C) * KH * KW);
+    return ternary ? 2 * kw : kw;
+}
+
+int64_t ftnn_pack_scratch_bytes(int N, int C, int H, int W, int ternary) {
+    return (int64_t)N * H * W * cpack_of(C) * (ternary ? 16 : 8);
+}
+
+int ftnn_quantize_im2row(int ternary, const float* d_x, const float* d_thr, int N, int C, int H,
+                         int W, int H_pad, int W_pad, int kH, int kW, int H_stride, int W_stride,
+                         int64_t* d_out, void* d_scratch, void* stream) {
+    int OH, OW;
+    int rc = check_conv_shape(N, C, H, W, H_pad, W_pad, kH, kW, H_stride, W_stride, &OH, &OW);
+    if (rc != FTNN_OK) return rc;
+    if (!d_x || !d_thr || !d_out || !d_scratch) return fail(FTNN_EINVAL, "null device pointer");
+    if (!aligned16(d_out) || !aligned16(d_scratch))
+        return fail(FTNN_EINVAL, "d_out and d_scratch must be 16-byte aligned");
+    hipError_t e = launch_quantize_im2row(ternary != 0, d_x, d_thr, N, C, H, W, H_pad, W_pad, kH,
+                                          kW, H_stride, W_stride, d_out, d_scratch,
+                                          (hipStream_t)stream);
+    return e == hipSuccess ? FTNN_OK : hip_fail(e, "quantize_im2row launch");
+}
+
+int ftnn_mm(int type, const int64_t* d_a, const int64_t* d_b, int N, int OH, int OW, int KN, int K,
+            int K_unpack, float prelu_alpha, float* d_y, void* stream) {
+    if (type < kTNN || type > kBNN) return fail(FTNN_EINVAL, "unknown network type %d", type);
+    if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0)
+        return fail(FTNN_EINVAL, "non-positive GEMM dimension");
+    if (!d_a || !d_b || !d_y) return fail(FTNN_EINVAL, "null device pointer");
+    if (!aligned16(d_a) || !aligned16(d_b))
+        return fail(FTNN_EINVAL, "GEMM operands must be 16-byte aligned");
+    const int64_t M = (int64_t)N * OH * OW;
+    if (M > 0x7fffffffLL || (int64_t)OH * OW > 0x7fffffffLL)
+        return fail(FTNN_EINVAL, "more than 2^31-1 output rows");
+    hipError_t e = launch_mm(type, d_a, d_b, M, OH * OW, KN, round4(K), K_unpack, prelu_alpha, d_y,
+                             (hipStream_t)stream);
+    return e == hipSuccess ? FTNN_OK : hip_fail(e, "mm launch");
+}
+
+int ftnn_conv(int type, const float* d_x, const float* d_thr, const int64_t* d_qw, int N, int C,
+              int H, int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride, int W_stride,
+              float prelu_alpha, int64_t* d_rows, void* d_scratch, float* d_y, void* stream) {
+    if (type < kTNN || type > kBNN) return fail(FTNN_EINVAL, "unknown network type %d", type);
+    int OH, OW;
+    int rc = check_conv_shape(N, C, H, W, H_pad, W_pad, KH, KW, H_stride, W_stride, &OH, &OW);
+    if (rc != FTNN_OK) return rc;
+    const int act_ternary = (type == kTNN || type == kTBN);
+    rc = ftnn_quantize_im2row(act_ternary, d_x, d_thr, N, C, H, W, H_pad, W_pad, KH, KW, H_stride,
+                              W_stride, d_rows, d_scratch, stream);
+    if (rc != FTNN_OK) return rc;
+    return ftnn_mm(type, d_rows, d_qw, N, OH, OW, KN, cpack_of(C) * KH * KW, C * KH * KW,
+                   prelu_alpha, d_y, stream);
+}
+
+int ftnn_pack_weights(int ternary, const float* d_w, const float* d_thr, int KN, int C, int KH,
+                      int KW, int64_t* d_out, void* stream) {
+    if (KN <= 0 || C <= 0 || KH <= 0 || KW <= 0) return fail(FTNN_EINVAL, "non-positive dimension");
+    if (!d_w || !d_thr || !d_out) return fail(FTNN_EINVAL, "null device pointer");
+    hipError_t e = launch_pack_weights(ternary != 0, d_w, d_thr, KN, C, KH, KW, d_out,
+                                       (hipStream_t)stream);
+    return e == hipSuccess ? FTNN_OK : hip_fail(e, "pack_weights launch");
+}
+
+int ftnn_pack_gemm_operand(const float* d_x, int I, int J, int64_t* d_out, void* stream) {
+    if (I <= 0 || J <= 0) return fail(FTNN_EINVAL, "non-positive dimension");
+    // the reference asserts the same (src/utils.c:258)
+    if (J % 256 != 0) return fail(FTNN_EINVAL, "J = %d is not a multiple of 256", J);
+    if (J / 64 / 4 > 65535) return fail(FTNN_EINVAL, "J = %d too large", J);
+    if (!d_x || !d_out) return fail(FTNN_EINVAL, "null device pointer");
+    hipError_t e = launch_pack_gemm_operand(d_x, I, J, d_out, (hipStream_t)stream);
+    return e == hipSuccess ? FTNN_OK : hip_fail(e, "pack_gemm_operand launch");
+}
+
+// ------------------------------------------------- reference entry points
+
+int64_t* t2r_p2_opt(float* x, float* q_thresholds, int N, int C, int H, int W, int H_pad, int W_pad,
+                    int kH, int kW, int H_stride, int W_stride) {
+    return host_quantize_im2row(true, x, q_thresholds, N, C, H, W, H_pad, W_pad, kH, kW, H_stride,
+                                W_stride);
+}
+
+int64_t* b2r(float* x, float* q_thresholds, int N, int C, int H, int W, int H_pad, int W_pad, int kH,
+             int kW, int H_stride, int W_stride) {
+    return host_quantize_im2row(false, x, q_thresholds, N, C, H, W, H_pad, W_pad, kH, kW, H_stride,
+                                W_stride);
+}
+
+float* mm_tnn(int64_t* a, int64_t* b, int N, int OH, int OW, int KN, int K, float prelu_alpha) {
+    return host_mm(kTNN, a, b, N, OH, OW, KN, K, 0, prelu_alpha);
+}
+float* mm_tbn(int64_t* a, int64_t* b, int N, int OH, int OW, int KN, int K, float prelu_alpha) {
+    return host_mm(kTBN, a, b, N, OH, OW, KN, K, 0, prelu_alpha);
+}
+float* mm_btn(int64_t* a, int64_t* b, int N, int OH, int OW, int KN, int K, float prelu_alpha) {
+    return host_mm(kBTN, a, b, N, OH, OW, KN, K, 0, prelu_alpha);
+}
+float* mm_bnn(int64_t* a, int64_t* b, int N, int OH, int OW, int KN, int K, int K_unpack,
+              float prelu_alpha) {
+    return host_mm(kBNN, a, b, N, OH, OW, KN, K, K_unpack, prelu_alpha);
+}
+
+void tnns_conv(testcase_t* t) {
+    const int type = (int)t->type;
+    const int N = t->batchcount, C = t->channelcount, H = t->inputH, W = t->inputW;
+    const int KN = t->kernelcount, KH = t->kernelH, KW = t->kernelW;
+    int OH, OW;
+    if (type < kTNN || type > kBNN) {
+        fail(FTNN_EINVAL, "unknown network type %d", type);
+        die("tnns_conv");
+    }
+    if (check_conv_shape(N, C, H, W, t->paddingH, t->paddingW, KH, KW, t->strideH, t->strideW, &OH,
+                         &OW) != FTNN_OK || KN <= 0)
+        die("tnns_conv");
+    const int act_tern = (type == kTNN || type == kTBN), w_tern = (type == kTNN || type == kBTN);
+    const size_t rows = (size_t)N * OH * OW;
+    float* d_x = (float*)upload(SLOT_X, t->input, (size_t)N * C * H * W * sizeof(float));
+    float* d_thr = (float*)upload(SLOT_THR, t->input_thresholds, (size_t)N * sizeof(float));
+    int64_t* d_w = (int64_t*)upload(SLOT_W, t->quantized_kernel_packing2,
+                                    (size_t)KN * ftnn_row_words(C, KH, KW, w_tern) * sizeof(int64_t));
+    int64_t* d_rows =
+        (int64_t*)dev_buf(SLOT_ROWS, rows * ftnn_row_words(C, KH, KW, act_tern) * sizeof(int64_t));
+    void* d_scr = dev_buf(SLOT_SCRATCH, (size_t)ftnn_pack_scratch_bytes(N, C, H, W, act_tern));
+    const size_t y_bytes = rows * KN * sizeof(float);
+    float* d_y = (float*)dev_buf(SLOT_Y, y_bytes);
+    if (ftnn_conv(type, d_x, d_thr, d_w, N, C, H, W, KN, KH, KW, t->paddingH, t->paddingW,
+                  t->strideH, t->strideW, t->preluAlpha, d_rows, d_scr, d_y,
+                  host_stream()) != FTNN_OK)
+        die("tnns_conv");
+    float* y = (float*)host_alloc(y_bytes, false);
+    download(y, d_y, y_bytes);
+    t->output = y;  // src/tnns/tnns_cpu_mm_p2.c:119
+}
+
+void tnns_gemm(testcase_tnns_gemm_t* t) {
+    // alpha is fixed to 1 (src/tnns/tnns_cpu_mm_p2.c:123)
+    float* result = mm_tnn(t->x_packing2, t->w_packing2, t->m, 1, 1, t->n, t->p_packed, 1.0f);
+    if (t->output) {
+        memcpy(t->output, result, (size_t)t->m * t->n * sizeof(float));
+        free(result);
+    } else {
+        t->output = result;
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,30 @@
+// Internal declarations shared by the kernel files and the C-ABI layer.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ftnn {
+
+constexpr int kTNN = 0, kTBN = 1, kBTN = 2, kBNN = 3;
+
+inline int cpack_of(int C) { return (C + 63) / 64; }
+inline int round4(int k) { return 4 * ((k + 3) / 4); }
+inline int out_dim(int in, int pad, int k, int stride) { return (in + 2 * pad - k) / stride + 1; }
+
+// record a failure text for ftnn_last_error(); returns `code`
+int fail(int code, const char* fmt, ...);
+
+// ---- pack_kernels.hip: launchers (arguments already validated) ----
+hipError_t launch_quantize_im2row(bool ternary, const float* d_x, const float* d_thr, int N, int C,
+                                  int H, int W, int H_pad, int W_pad, int kH, int kW, int H_stride,
+                                  int W_stride, int64_t* d_out, void* d_scratch, hipStream_t st);
+hipError_t launch_pack_weights(bool ternary, const float* d_w, const float* d_thr, int KN, int C,
+                               int KH, int KW, int64_t* d_out, hipStream_t st);
+hipError_t launch_pack_gemm_operand(const float* d_x, int I, int J, int64_t* d_out, hipStream_t st);
+
+// ---- mm_kernels.hip ----
+hipError_t launch_mm(int type, const int64_t* d_a, const int64_t* d_b, int64_t M, int OHW, int KN,
+                     int Kw /* words per plane, multiple of 4 */, int K_unpack, float alpha,
+                     float* d_y, hipStream_t st);
+
+}  // namespace ftnn

@@ -1,0 +1,269 @@
+// Quantise / bit-pack / im2row kernels (gfx950).
+//
+// Activations (t2r_p2_opt, src/tnns/ternarize2row_avx2.c:715-803; b2r,
+// src/tnns/binarize2row_avx2.c:131-199) are produced in two HBM-bound steps:
+//
+//   1. quantise: fp32 NCHW -> channel-packed pixels P[n][pixel][ic], one 64-bit
+//      word per plane for 64 channels.  The input is read exactly once.  Two
+//      forms: lanes along pixels (coalesced reads of each channel plane, every
+//      lane assembles its own word), and, for 1x1 spatial inputs and row-major
+//      GEMM operands where 64 consecutive floats ARE one word, one wavefront
+//      ballot per word.
+//   2. im2row: a gather of 64-bit words from P into the Packing-2 row layout,
+//      one work-item per output word, with the fill rules of the reference for
+//      everything not backed by a real (pixel, channel).
+//
+// Weights (ternarize_opt_avx2 / binarize_opt_avx2, src/utils.c:468-521,634-675)
+// and GEMM operands (bitpacking2, src/utils.c:257-291) are packed by their own
+// kernels; they are offline work in the reference and are not tuned here.
+#include "ftnn_internal.h"
+
+namespace ftnn {
+
+namespace {
+
+// position of word idx of plane `plane` in a Packing-2 row
+// (src/tnns/ternarize2row_avx2.c:464-469)
+__device__ __forceinline__ int64_t p2_pos(int64_t idx, int plane) {
+    return (idx >> 2) * 8 + (idx & 3) + (plane ? 4 : 0);
+}
+
+// ---------------------------------------------------------------- quantise
+// lanes along pixels: grid (ceil(HW/256), C_pack, N)
+template <bool TERN>
+__global__ __launch_bounds__(256) void k_quantize_pixels(const float* __restrict__ x,
+                                                         const float* __restrict__ thr, int C,
+                                                         int HW, int CP,
+                                                         unsigned long long* __restrict__ P) {
+    const int p = blockIdx.x * 256 + threadIdx.x;
+    const int ic = blockIdx.y, n = blockIdx.z;
+    if (p >= HW) return;
+    const float t = thr[n];
+    const int nb = min(64, C - ic * 64);
+    const float* xp = x + ((size_t)n * C + (size_t)ic * 64) * HW + p;
+    uint32_t neg[2] = {0u, 0u}, nz[2] = {0u, 0u};
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+#pragma unroll 8
+        for (int bit = 0; bit < 32; bit++) {
+            const int c = half * 32 + bit;
+            if (c < nb) {
+                const float v = xp[(size_t)c * HW];
+                if (TERN) {
+                    // strict compares, src/tnns/ternarize2row_avx2.c:443-449
+                    const bool isneg = v < -t;
+                    const bool ispos = v > t;
+                    neg[half] |= (isneg ? 1u : 0u) << bit;
+                    nz[half] |= ((isneg || ispos) ? 1u : 0u) << bit;
+                } else {
+                    // src/tnns/binarize2row_avx2.c:19-21
+                    neg[half] |= (v < t ? 1u : 0u) << bit;
+                }
+            }
+        }
+    }
+    const size_t o = ((size_t)n * HW + p) * CP + ic;
+    const unsigned long long s = ((unsigned long long)neg[1] << 32) | neg[0];
+    if (TERN) {
+        const unsigned long long z = ~(((unsigned long long)nz[1] << 32) | nz[0]);
+        reinterpret_cast<ulonglong2*>(P)[o] = make_ulonglong2(s, z);
+    } else {
+        P[o] = s;
+    }
+}
+
+// One wavefront ballot per 64-bit word: rows of J consecutive floats.
+// MODE 0: ternary thresholds, 1: binary threshold, 2: exact values {-1,0,+1}
+// (bitpacking2).  P2ROW: write straight into Packing-2 rows of 2*J/64 words
+// instead of the (sign, zero) pair array.  grid (R, ceil(words/4)), block 256.
+template <int MODE, bool P2ROW>
+__global__ __launch_bounds__(256) void k_quantize_ballot(const float* __restrict__ x,
+                                                         const float* __restrict__ thr, int J,
+                                                         int words,
+                                                         unsigned long long* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int wd = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int r = blockIdx.x;
+    if (wd >= words) return;  // uniform per wavefront
+    const int j = wd * 64 + lane;
+    const bool in = j < J;
+    const float v = in ? x[(size_t)r * J + j] : 0.0f;
+    bool isneg, isnz;
+    if (MODE == 0) {
+        const float t = thr[r];
+        isneg = in && v < -t;
+        isnz = in && (isneg || v > t);
+    } else if (MODE == 1) {
+        isneg = in && v < thr[r];
+        isnz = true;
+    } else {
+        isneg = v == -1.0f;
+        isnz = !(v == 0.0f);
+    }
+    const unsigned long long s = __ballot(isneg);
+    const unsigned long long z = ~__ballot(isnz);
+    if (lane == 0) {
+        if (P2ROW) {
+            unsigned long long* row = out + (size_t)r * 2 * words;
+            row[p2_pos(wd, 0)] = s;
+            row[p2_pos(wd, 1)] = z;
+        } else if (MODE == 1) {
+            out[(size_t)r * words + wd] = s;
+        } else {
+            reinterpret_cast<ulonglong2*>(out)[(size_t)r * words + wd] = make_ulonglong2(s, z);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ im2row
+// one work-item per output word (pair); lanes run along the row
+template <bool TERN>
+__global__ __launch_bounds__(256) void k_im2row(const unsigned long long* __restrict__ P, int H,
+                                                int W, int CP, int OH, int OW, int KW, int K,
+                                                int Kw, int H_pad, int W_pad, int H_stride,
+                                                int W_stride, int64_t total,
+                                                unsigned long long* __restrict__ out) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= total) return;
+    const int64_t r = e / Kw;
+    const int idx = (int)(e - r * Kw);
+    unsigned long long s = 0ull, z = ~0ull;
+    if (idx < K) {
+        const int ic = idx % CP, tap = idx / CP;
+        const int kh = tap / KW, kw = tap - kh * KW;
+        const int ow = (int)(r % OW);
+        const int64_t t2 = r / OW;
+        const int oh = (int)(t2 % OH);
+        const int64_t n = t2 / OH;
+        const int ih = oh * H_stride + kh - H_pad, iw = ow * W_stride + kw - W_pad;
+        if (ih >= 0 && ih < H && iw >= 0 && iw < W) {
+            const size_t o = ((size_t)n * H * W + (size_t)ih * W + iw) * CP + ic;
+            if (TERN) {
+                const ulonglong2 v = reinterpret_cast<const ulonglong2*>(P)[o];
+                s = v.x;
+                z = v.y;
+            } else {
+                s = P[o];
+            }
+        }
+    }
+    if (TERN) {
+        unsigned long long* row = out + (size_t)r * 2 * Kw;
+        row[p2_pos(idx, 0)] = s;
+        row[p2_pos(idx, 1)] = z;
+    } else {
+        out[(size_t)r * Kw + idx] = s;
+    }
+}
+
+// ------------------------------------------------------------- weight packers
+// one work-item per output word; w is fp32 (KN, C, KH, KW)
+template <bool TERN>
+__global__ __launch_bounds__(256) void k_pack_weights(const float* __restrict__ w,
+                                                      const float* __restrict__ thr, int C,
+                                                      int taps, int CP, int K, int Kw,
+                                                      int64_t total,
+                                                      unsigned long long* __restrict__ out) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= total) return;
+    const int64_t n = e / Kw;
+    const int idx = (int)(e - n * Kw);
+    unsigned long long s = 0ull, z = TERN ? ~0ull : 0ull;
+    if (idx < K) {
+        const int ic = idx % CP, tap = idx / CP;
+        const float t = thr[n];
+        z = 0ull;
+        for (int bit = 0; bit < 64; bit++) {
+            const int c = ic * 64 + bit;
+            if (TERN) {
+                // channels past C read as 0.0 and take the same compares, positive side
+                // first (src/utils.c:498-509)
+                const float v = c < C ? w[((size_t)n * C + c) * taps + tap] : 0.0f;
+                if (v > t) {
+                } else if (v < -t) {
+                    s |= 1ull << bit;
+                } else {
+                    z |= 1ull << bit;
+                }
+            } else if (c < C) {
+                // src/utils.c:654-660
+                const float v = w[((size_t)n * C + c) * taps + tap];
+                if (v < t) s |= 1ull << bit;
+            }
+        }
+    }
+    if (TERN) {
+        unsigned long long* row = out + (size_t)n * 2 * Kw;
+        row[p2_pos(idx, 0)] = s;
+        row[p2_pos(idx, 1)] = z;
+    } else {
+        out[(size_t)n * Kw + idx] = s;
+    }
+}
+
+}  // namespace
+
+hipError_t launch_quantize_im2row(bool ternary, const float* d_x, const float* d_thr, int N, int C,
+                                  int H, int W, int H_pad, int W_pad, int kH, int kW, int H_stride,
+                                  int W_stride, int64_t* d_out, void* d_scratch, hipStream_t st) {
+    const int CP = cpack_of(C), HW = H * W;
+    const int OH = out_dim(H, H_pad, kH, H_stride), OW = out_dim(W, W_pad, kW, W_stride);
+    const int K = CP * kH * kW, Kw = round4(K);
+    unsigned long long* P = static_cast<unsigned long long*>(d_scratch);
+    if (HW == 1) {
+        // 64 consecutive floats are one word: wavefront ballot
+        dim3 grid(N, (CP + 3) / 4);
+        if (ternary)
+            hipLaunchKernelGGL((k_quantize_ballot<0, false>), grid, dim3(256), 0, st, d_x, d_thr, C,
+                               CP, P);
+        else
+            hipLaunchKernelGGL((k_quantize_ballot<1, false>), grid, dim3(256), 0, st, d_x, d_thr, C,
+                               CP, P);
+    } else {
+        dim3 grid((HW + 255) / 256, CP, N);
+        if (ternary)
+            hipLaunchKernelGGL((k_quantize_pixels<true>), grid, dim3(256), 0, st, d_x, d_thr, C, HW,
+                               CP, P);
+        else
+            hipLaunchKernelGGL((k_quantize_pixels<false>), grid, dim3(256), 0, st, d_x, d_thr, C,
+                               HW, CP, P);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const int64_t total = (int64_t)N * OH * OW * Kw;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    unsigned long long* out = reinterpret_cast<unsigned long long*>(d_out);
+    if (ternary)
+        hipLaunchKernelGGL((k_im2row<true>), dim3(blocks), dim3(256), 0, st, P, H, W, CP, OH, OW, kW,
+                           K, Kw, H_pad, W_pad, H_stride, W_stride, total, out);
+    else
+        hipLaunchKernelGGL((k_im2row<false>), dim3(blocks), dim3(256), 0, st, P, H, W, CP, OH, OW,
+                           kW, K, Kw, H_pad, W_pad, H_stride, W_stride, total, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_pack_weights(bool ternary, const float* d_w, const float* d_thr, int KN, int C,
+                               int KH, int KW, int64_t* d_out, hipStream_t st) {
+    const int CP = cpack_of(C), K = CP * KH * KW, Kw = round4(K);
+    const int64_t total = (int64_t)KN * Kw;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    unsigned long long* out = reinterpret_cast<unsigned long long*>(d_out);
+    if (ternary)
+        hipLaunchKernelGGL((k_pack_weights<true>), dim3(blocks), dim3(256), 0, st, d_w, d_thr, C,
+                           KH * KW, CP, K, Kw, total, out);
+    else
+        hipLaunchKernelGGL((k_pack_weights<false>), dim3(blocks), dim3(256), 0, st, d_w, d_thr, C,
+                           KH * KW, CP, K, Kw, total, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_pack_gemm_operand(const float* d_x, int I, int J, int64_t* d_out, hipStream_t st) {
+    const int words = J / 64;
+    dim3 grid(I, (words + 3) / 4);
+    hipLaunchKernelGGL((k_quantize_ballot<2, true>), grid, dim3(256), 0, st, d_x,
+                       (const float*)nullptr, J, words,
+                       reinterpret_cast<unsigned long long*>(d_out));
+    return hipGetLastError();
+}
+
+}  // namespace ftnn

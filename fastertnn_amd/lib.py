@@ -1,0 +1,236 @@
+"""ctypes binding of libftnn_hip.so (the C ABI declared in include/ftnn.h).
+
+Device-memory entry points take torch CUDA tensors (used only as device buffers)
+and run on torch's current stream.  Host-memory entry points are the reference's
+own (`tnns_conv`, `tnns_gemm`, `t2r_p2_opt`, `b2r`, `mm_*`): they take numpy
+arrays, and the heap buffer each one returns is copied into numpy and freed, as a
+C caller would free it.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import TNN, TBN, BTN, BNN, act_is_ternary, weight_is_ternary
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libftnn_hip.so")
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError("%s is missing: build it with `python -m fastertnn_amd.build` "
+                      "(there is no CPU fallback)" % LIB_PATH)
+
+_L = C.CDLL(LIB_PATH)
+_libc = C.CDLL(None)
+_libc.free.argtypes = [C.c_void_p]
+
+_vp = C.c_void_p
+_L.ftnn_last_error.restype = C.c_char_p
+_L.ftnn_version.restype = C.c_char_p
+_L.ftnn_row_words.restype = C.c_int64
+_L.ftnn_pack_scratch_bytes.restype = C.c_int64
+_L.ftnn_quantize_im2row.argtypes = [C.c_int, _vp, _vp] + [C.c_int] * 10 + [_vp, _vp, _vp]
+_L.ftnn_mm.argtypes = [C.c_int, _vp, _vp] + [C.c_int] * 6 + [C.c_float, _vp, _vp]
+_L.ftnn_conv.argtypes = [C.c_int, _vp, _vp, _vp] + [C.c_int] * 11 + [C.c_float, _vp, _vp, _vp, _vp]
+_L.ftnn_pack_weights.argtypes = [C.c_int, _vp, _vp] + [C.c_int] * 4 + [_vp, _vp]
+_L.ftnn_pack_gemm_operand.argtypes = [_vp, C.c_int, C.c_int, _vp, _vp]
+for _n in ("t2r_p2_opt", "b2r"):
+    getattr(_L, _n).restype = _vp
+    getattr(_L, _n).argtypes = [_vp, _vp] + [C.c_int] * 10
+for _n in ("mm_tnn", "mm_tbn", "mm_btn"):
+    getattr(_L, _n).restype = _vp
+    getattr(_L, _n).argtypes = [_vp, _vp] + [C.c_int] * 5 + [C.c_float]
+_L.mm_bnn.restype = _vp
+_L.mm_bnn.argtypes = [_vp, _vp] + [C.c_int] * 6 + [C.c_float]
+_L.tnns_conv.restype = None
+_L.tnns_gemm.restype = None
+
+EXPORTS = ("tnns_conv", "tnns_gemm", "t2r_p2_opt", "b2r", "mm_tnn", "mm_tbn", "mm_btn", "mm_bnn",
+           "ftnn_last_error", "ftnn_version", "ftnn_out_dim", "ftnn_row_words",
+           "ftnn_pack_scratch_bytes", "ftnn_quantize_im2row", "ftnn_mm", "ftnn_conv",
+           "ftnn_pack_weights", "ftnn_pack_gemm_operand")
+
+
+class FtnnError(RuntimeError):
+    pass
+
+
+def _check(rc):
+    if rc != 0:
+        raise FtnnError("ftnn error %d: %s" % (rc, _L.ftnn_last_error().decode()))
+
+
+def version():
+    return _L.ftnn_version().decode()
+
+
+def out_dim(n, pad, k, stride):
+    return int(_L.ftnn_out_dim(n, pad, k, stride))
+
+
+def row_words(c, kh, kw, ternary):
+    return int(_L.ftnn_row_words(c, kh, kw, int(ternary)))
+
+
+def pack_scratch_bytes(n, c, h, w, ternary):
+    return int(_L.ftnn_pack_scratch_bytes(n, c, h, w, int(ternary)))
+
+
+# ------------------------------------------------------------ device entry points
+
+def _stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t, dtype=None):
+    import torch
+    assert t.is_cuda and t.is_contiguous(), "expected a contiguous CUDA tensor"
+    if dtype is not None:
+        assert t.dtype == dtype, "expected %s, got %s" % (dtype, t.dtype)
+    return t.data_ptr()
+
+
+def quantize_im2row(x, thr, kh, kw, pad, stride, ternary, out=None, scratch=None):
+    """t2r_p2_opt (ternary) / b2r (binary) on device tensors; returns int64 rows."""
+    import torch
+    n, c, h, w = x.shape
+    oh, ow = out_dim(h, pad, kh, stride), out_dim(w, pad, kw, stride)
+    if oh <= 0 or ow <= 0:
+        raise FtnnError("kernel larger than padded input")
+    words = row_words(c, kh, kw, ternary)
+    if out is None:
+        out = torch.empty(n * oh * ow * words, dtype=torch.int64, device=x.device)
+    if scratch is None:
+        scratch = torch.empty(pack_scratch_bytes(n, c, h, w, ternary), dtype=torch.uint8, device=x.device)
+    _check(_L.ftnn_quantize_im2row(int(ternary), _dev(x, torch.float32), _dev(thr, torch.float32),
+                                   n, c, h, w, pad, pad, kh, kw, stride, stride, _dev(out), _dev(scratch),
+                                   _stream()))
+    return out
+
+
+def mm(typ, a, b, n, oh, ow, kn, k, alpha, k_unpack=0, out=None):
+    """mm_tnn / mm_tbn / mm_btn / mm_bnn on device tensors; returns fp32 (n, kn, oh, ow)."""
+    import torch
+    if out is None:
+        out = torch.empty((n, kn, oh, ow), dtype=torch.float32, device=a.device)
+    _check(_L.ftnn_mm(typ, _dev(a), _dev(b), n, oh, ow, kn, k, k_unpack, alpha, _dev(out, torch.float32),
+                      _stream()))
+    return out
+
+
+def conv(typ, x, thr, qw, kn, kh, kw, pad, stride, alpha, rows=None, scratch=None, out=None):
+    """One conv layer (tnn_conv_p2 & co.) on device tensors."""
+    import torch
+    n, c, h, w = x.shape
+    oh, ow = out_dim(h, pad, kh, stride), out_dim(w, pad, kw, stride)
+    if oh <= 0 or ow <= 0:
+        raise FtnnError("kernel larger than padded input")
+    tern = act_is_ternary(typ)
+    if rows is None:
+        rows = torch.empty(n * oh * ow * row_words(c, kh, kw, tern), dtype=torch.int64, device=x.device)
+    if scratch is None:
+        scratch = torch.empty(pack_scratch_bytes(n, c, h, w, tern), dtype=torch.uint8, device=x.device)
+    if out is None:
+        out = torch.empty((n, kn, oh, ow), dtype=torch.float32, device=x.device)
+    _check(_L.ftnn_conv(typ, _dev(x, torch.float32), _dev(thr, torch.float32), _dev(qw), n, c, h, w, kn, kh,
+                        kw, pad, pad, stride, stride, alpha, _dev(rows), _dev(scratch),
+                        _dev(out, torch.float32), _stream()))
+    return out
+
+
+def pack_weights(w, thr, ternary):
+    """ternarize_opt_avx2 / binarize_opt_avx2 on device tensors."""
+    import torch
+    kn, c, kh, kw = w.shape
+    out = torch.empty(kn * row_words(c, kh, kw, ternary), dtype=torch.int64, device=w.device)
+    _check(_L.ftnn_pack_weights(int(ternary), _dev(w, torch.float32), _dev(thr, torch.float32), kn, c, kh, kw,
+                                _dev(out), _stream()))
+    return out
+
+
+def pack_gemm_operand(x):
+    """bitpacking2 on a device tensor [I][J] of {-1,0,+1} floats."""
+    import torch
+    i, j = x.shape
+    out = torch.empty(max(i * j // 32, 1), dtype=torch.int64, device=x.device)
+    _check(_L.ftnn_pack_gemm_operand(_dev(x, torch.float32), i, j, _dev(out), _stream()))
+    return out
+
+
+# -------------------------------------------------- reference (host) entry points
+
+class Testcase(C.Structure):
+    """testcase_t, include/tnns/data.h:4-25."""
+    _fields_ = [("type", C.c_int), ("batchcount", C.c_int), ("channelcount", C.c_int),
+                ("inputW", C.c_int), ("inputH", C.c_int), ("kernelcount", C.c_int),
+                ("kernelW", C.c_int), ("kernelH", C.c_int), ("paddingW", C.c_int),
+                ("paddingH", C.c_int), ("strideW", C.c_int), ("strideH", C.c_int),
+                ("preluAlpha", C.c_float), ("input_thresholds", _vp), ("input", _vp),
+                ("kernel", _vp), ("quantized_kernel_packing0", _vp),
+                ("quantized_kernel_packing1", _vp), ("quantized_kernel_packing2", _vp),
+                ("output", _vp)]
+
+
+class TestcaseGemm(C.Structure):
+    """testcase_tnns_gemm_t, include/tnns/data.h:27-41."""
+    _fields_ = [("m", C.c_int), ("p", C.c_int), ("p_packed", C.c_int), ("n", C.c_int),
+                ("x", _vp), ("w", _vp), ("x_packing0", _vp), ("x_packing1", _vp), ("x_packing2", _vp),
+                ("w_packing0", _vp), ("w_packing1", _vp), ("w_packing2", _vp), ("output", _vp)]
+
+
+def _take(ptr, n, dtype):
+    buf = (C.c_char * (n * np.dtype(dtype).itemsize)).from_address(ptr)
+    out = np.frombuffer(buf, dtype=dtype).copy()
+    _libc.free(ptr)
+    return out
+
+
+def _np(a, dtype):
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def host_quantize_im2row(x, thr, kh, kw, pad, stride, ternary):
+    x, thr = _np(x, np.float32), _np(thr, np.float32)
+    n, c, h, w = x.shape
+    oh, ow = out_dim(h, pad, kh, stride), out_dim(w, pad, kw, stride)
+    fn = _L.t2r_p2_opt if ternary else _L.b2r
+    ptr = fn(x.ctypes.data, thr.ctypes.data, n, c, h, w, pad, pad, kh, kw, stride, stride)
+    return _take(ptr, n * oh * ow * row_words(c, kh, kw, ternary), np.int64)
+
+
+def host_mm(typ, a, b, n, oh, ow, kn, k, alpha, k_unpack=0):
+    a, b = _np(a, np.int64), _np(b, np.int64)
+    if typ == BNN:
+        ptr = _L.mm_bnn(a.ctypes.data, b.ctypes.data, n, oh, ow, kn, k, k_unpack, alpha)
+    else:
+        fn = (_L.mm_tnn, _L.mm_tbn, _L.mm_btn)[typ]
+        ptr = fn(a.ctypes.data, b.ctypes.data, n, oh, ow, kn, k, alpha)
+    return _take(ptr, n * kn * oh * ow, np.float32).reshape(n, kn, oh, ow)
+
+
+def host_conv(typ, x, thr, qw, kn, kh, kw, pad, stride, alpha):
+    """tnns_conv on a testcase_t built from numpy arrays."""
+    x, thr, qw = _np(x, np.float32), _np(thr, np.float32), _np(qw, np.int64)
+    n, c, h, w = x.shape
+    t = Testcase(type=typ, batchcount=n, channelcount=c, inputW=w, inputH=h, kernelcount=kn, kernelW=kw,
+                 kernelH=kh, paddingW=pad, paddingH=pad, strideW=stride, strideH=stride, preluAlpha=alpha,
+                 input_thresholds=thr.ctypes.data, input=x.ctypes.data,
+                 quantized_kernel_packing2=qw.ctypes.data)
+    _L.tnns_conv(C.byref(t))
+    oh, ow = out_dim(h, pad, kh, stride), out_dim(w, pad, kw, stride)
+    return _take(t.output, n * kn * oh * ow, np.float32).reshape(n, kn, oh, ow)
+
+
+def host_gemm(xp, wp, m, n, p_packed, into=None):
+    """tnns_gemm; `into` (m x n float32) exercises the copy-into-output branch."""
+    xp, wp = _np(xp, np.int64), _np(wp, np.int64)
+    t = TestcaseGemm(m=m, p=p_packed * 64, p_packed=p_packed, n=n, x_packing2=xp.ctypes.data,
+                     w_packing2=wp.ctypes.data)
+    if into is not None:
+        assert into.dtype == np.float32 and into.size == m * n and into.flags.c_contiguous
+        t.output = into.ctypes.data
+        _L.tnns_gemm(C.byref(t))
+        return into
+    _L.tnns_gemm(C.byref(t))
+    return _take(t.output, m * n, np.float32).reshape(m, n)

@@ -1,0 +1,179 @@
+/*
+ * ftnn.h -- C ABI of libftnn_hip.so, the MI355X (gfx950) implementation of the
+ * FasterTNN ternary/binary inference hot path.
+ *
+ * Two layers:
+ *
+ *  1. The reference's own entry points, same names, argument meaning, struct
+ *     layout and ownership rules, so that the reference's layer drivers link
+ *     against this library instead of its tnns_cpu_mm_p2.o / mm_p2_final_*.o /
+ *     ternarize2row_*.o / binarize2row_*.o objects.  They take and return host
+ *     memory; every returned buffer is ordinary heap memory that the caller
+ *     free()s.  Failure handling follows the reference: a message on stderr and
+ *     abort().
+ *
+ *  2. ftnn_* entry points that work on device memory and a caller-supplied HIP
+ *     stream (passed as void*, 0 = the null stream).  They return 0 on success
+ *     and a negative FTNN_E* code otherwise; ftnn_last_error() gives the text.
+ *     They never synchronise the stream.
+ *
+ * Paths in the comments are relative to the reference tree.
+ */
+#ifndef FTNN_H
+#define FTNN_H
+
+#include <stdint.h>
+
+/* symbols exported by the shared library */
+#define FTNN_API __attribute__((visibility("default")))
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ types */
+
+/* include/tnns/common.h:16 */
+enum tnns_type { TNN, TBN, BTN, BNN };
+
+/* include/tnns/data.h:4-25 (112 bytes on LP64; field order is part of the ABI) */
+typedef struct testcase {
+    enum tnns_type type;
+    int batchcount;
+    int channelcount;
+    int inputW;
+    int inputH;
+    int kernelcount;
+    int kernelW;
+    int kernelH;
+    int paddingW;
+    int paddingH;
+    int strideW;
+    int strideH;
+    float preluAlpha;
+    float *input_thresholds;            /* one threshold per batch item      */
+    float *input;                       /* fp32 NCHW                         */
+    float *kernel;                      /* fp32 (KN,C,KH,KW); unused here    */
+    int64_t *quantized_kernel_packing0; /* unused here                       */
+    int64_t *quantized_kernel_packing1; /* unused here                       */
+    int64_t *quantized_kernel_packing2; /* Packing-2 weights (host)          */
+    float *output;                      /* overwritten with a fresh buffer   */
+} testcase_t;
+
+/* include/tnns/data.h:27-41 (88 bytes on LP64) */
+typedef struct testcase_tnns_gemm {
+    int m;
+    int p;
+    int p_packed;
+    int n;
+    float *x;
+    float *w;
+    int64_t *x_packing0;
+    int64_t *x_packing1;
+    int64_t *x_packing2;
+    int64_t *w_packing0;
+    int64_t *w_packing1;
+    int64_t *w_packing2;
+    float *output;
+} testcase_tnns_gemm_t;
+
+/* ------------------------------------- 1. reference entry points (host memory) */
+
+/* include/tnns/tnns_cpu.h:4, src/tnns/tnns_cpu_mm_p2.c:83-120.  Runs one conv layer
+ * of data->type; data->output is replaced by a malloc'd fp32 NCHW tensor. */
+FTNN_API void tnns_conv(testcase_t *data);
+
+/* include/tnns/tnns_cpu.h:6, src/tnns/tnns_cpu_mm_p2.c:122-133.  TNN GEMM of the
+ * Packing-2 operands with alpha = 1; copies into data->output when it is set,
+ * otherwise hands over a malloc'd m x n matrix. */
+FTNN_API void tnns_gemm(testcase_tnns_gemm_t *data);
+
+/* include/tnns/ternarize2row.h:7, src/tnns/ternarize2row_avx2.c:715-803.
+ * Ternarise + im2row + Packing 2; returns aligned_alloc(32, ...) memory. */
+FTNN_API int64_t *t2r_p2_opt(float *x, float *q_thresholds, int N, int C, int H, int W, int H_pad,
+                    int W_pad, int kH, int kW, int H_stride, int W_stride);
+
+/* include/tnns/binarize2row.h:4, src/tnns/binarize2row_avx2.c:131-199. */
+FTNN_API int64_t *b2r(float *x, float *q_thresholds, int N, int C, int H, int W, int H_pad, int W_pad,
+             int kH, int kW, int H_stride, int W_stride);
+
+/* include/tnns/mm.h:5-8; src/tnns/mm_p2_final_{tnn,tbn,btn,bnn}_avx2.c.  K is the
+ * number of 64-bit words per plane before rounding up to a multiple of 4.  The
+ * result is malloc'd fp32 in (N, KN, OH, OW) order with PReLU(alpha) applied. */
+FTNN_API float *mm_tnn(int64_t *a, int64_t *b, int N, int OH, int OW, int KN, int K, float prelu_alpha);
+FTNN_API float *mm_tbn(int64_t *a, int64_t *b, int N, int OH, int OW, int KN, int K, float prelu_alpha);
+FTNN_API float *mm_btn(int64_t *a, int64_t *b, int N, int OH, int OW, int KN, int K, float prelu_alpha);
+FTNN_API float *mm_bnn(int64_t *a, int64_t *b, int N, int OH, int OW, int KN, int K, int K_unpack,
+              float prelu_alpha);
+
+/* ------------------------------------------- 2. device-memory entry points */
+
+#define FTNN_OK 0
+#define FTNN_EINVAL (-1)  /* bad argument (shape, alignment, null pointer) */
+#define FTNN_EHIP (-2)    /* a HIP call failed                              */
+#define FTNN_ENOMEM (-3)  /* device or host allocation failed               */
+
+/* text of the last failure on the calling thread ("" if none) */
+FTNN_API const char *ftnn_last_error(void);
+
+/* library version string, e.g. "ftnn-hip 0.1 gfx950" */
+FTNN_API const char *ftnn_version(void);
+
+/* OH = (in + 2*pad - k)/stride + 1 (src/tnns/tnns_cpu_mm_p2.c:7-10) */
+FTNN_API int ftnn_out_dim(int in, int pad, int k, int stride);
+
+/* int64 words in one packed row: round4(ceil(C/64)*KH*KW), twice that for a
+ * ternary (two-plane) row (src/tnns/ternarize2row_avx2.c:730-732) */
+FTNN_API int64_t ftnn_row_words(int C, int KH, int KW, int ternary);
+
+/* Device scratch, in bytes, that ftnn_quantize_im2row / ftnn_conv need for the
+ * channel-packed copy of the input (N*H*W*ceil(C/64) words per plane). */
+FTNN_API int64_t ftnn_pack_scratch_bytes(int N, int C, int H, int W, int ternary);
+
+/*
+ * Quantise + im2row + bit-pack on the device: the work of t2r_p2_opt (ternary != 0,
+ * src/tnns/ternarize2row_avx2.c:715-803) or b2r (ternary == 0,
+ * src/tnns/binarize2row_avx2.c:131-199).  d_x fp32 NCHW, d_thr[N], d_out holds
+ * N*OH*OW rows of ftnn_row_words() words, d_scratch holds
+ * ftnn_pack_scratch_bytes() bytes.
+ */
+FTNN_API int ftnn_quantize_im2row(int ternary, const float *d_x, const float *d_thr, int N, int C, int H,
+                         int W, int H_pad, int W_pad, int kH, int kW, int H_stride, int W_stride,
+                         int64_t *d_out, void *d_scratch, void *stream);
+
+/*
+ * Popcount GEMM + PReLU on the device for type TNN/TBN/BTN/BNN
+ * (src/tnns/mm_p2_final_{tnn,tbn,btn,bnn}_avx2.c).  d_a: N*OH*OW packed rows,
+ * d_b: KN packed rows, d_y: fp32 (N,KN,OH,OW).  K_unpack is read for BNN only.
+ * Both operands must be 16-byte aligned.
+ */
+FTNN_API int ftnn_mm(int type, const int64_t *d_a, const int64_t *d_b, int N, int OH, int OW, int KN,
+            int K, int K_unpack, float prelu_alpha, float *d_y, void *stream);
+
+/*
+ * One conv layer on the device: ftnn_quantize_im2row then ftnn_mm
+ * (src/tnns/tnns_cpu_mm_p2.c:6-80).  d_rows holds N*OH*OW packed rows.
+ */
+FTNN_API int ftnn_conv(int type, const float *d_x, const float *d_thr, const int64_t *d_qw, int N, int C,
+              int H, int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride,
+              int W_stride, float prelu_alpha, int64_t *d_rows, void *d_scratch, float *d_y,
+              void *stream);
+
+/*
+ * Weight packers on the device: fp32 (KN,C,KH,KW) -> Packing-2 rows.  ternary != 0 is
+ * ternarize_opt_avx2 (src/utils.c:468-521), ternary == 0 is binarize_opt_avx2
+ * (src/utils.c:634-675).  d_thr[KN].
+ */
+FTNN_API int ftnn_pack_weights(int ternary, const float *d_w, const float *d_thr, int KN, int C, int KH,
+                      int KW, int64_t *d_out, void *stream);
+
+/*
+ * GEMM operand packer on the device: fp32 row-major [I][J] with values in
+ * {-1,0,+1} -> Packing 2 (bitpacking2, src/utils.c:257-291).  J % 256 must be 0.
+ */
+FTNN_API int ftnn_pack_gemm_operand(const float *d_x, int I, int J, int64_t *d_out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FTNN_H */
