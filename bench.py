@@ -1,0 +1,228 @@
+#!/usr/bin/env python3
+"""Benchmark of the TNN hot path on one MI355X.
+
+Headline workload: the large compute-bound TNN GEMM (M = N = 8192, K = 32768,
+uniform ternary operands in Packing 2, PReLU(0.5) fused).  One "step" is one call
+of the GEMM entry point of the C ABI (`ftnn_mm`) with both packed operands and
+the output resident in HBM.  Prints ONE JSON line:
+
+  value        ternary GMAC/s = M*N*K / time
+  roofline     vector-ALU roofline of the GEMM kernel: algorithmic lane-ops per
+               launch (4 VALU ops per pair of 32-lane dwords for TNN) over the
+               HIP-event duration of the launches, against 256 CU x 4 SIMD x 16
+               lanes x 2.4 GHz
+  cpu_baseline the reference's own AVX2 GEMM (compiled from its sources into
+               oracle/_ref) on one host core over a bounded row sample of the same
+               operands; the GPU rows of that sample are compared bit-for-bit
+  extra        conv-layer latencies (kernel-only and host-pointer ABI inclusive)
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+VALU_PEAK_TOPS = 256 * 4 * 16 * 2.4e9 / 1e12  # 39.32 T lane-ops/s (int32 VALU, one op per lane per clock)
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--m", type=int, default=8192)
+    ap.add_argument("--n", type=int, default=8192)
+    ap.add_argument("--k", type=int, default=32768)
+    ap.add_argument("--cpu-rows", type=int, default=8192, help="rows of A in the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--no-extra", action="store_true", help="skip the conv-layer latency section")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 256 MiB device copy, the known-size dispatch that "
+                         "FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
+    return ap.parse_args()
+
+
+def ternary_operand(torch, lib, rows, k, seed):
+    """uniform {-1,0,+1} fp32 [rows][k] generated on the device, packed by the library"""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    out = torch.empty(rows * k // 32, dtype=torch.int64, device="cuda")
+    step = max(1, (1 << 28) // k)  # <= 1 GiB of fp32 at a time
+    for r0 in range(0, rows, step):
+        r1 = min(rows, r0 + step)
+        x = torch.randint(-1, 2, (r1 - r0, k), generator=g, device="cuda", dtype=torch.int8).float()
+        out[r0 * k // 32:r1 * k // 32] = lib.pack_gemm_operand(x)
+    return out
+
+
+def event_times(torch, fn, reps):
+    """per-launch duration in ms from HIP events recorded on the launch stream"""
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for a, b in ev:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return [a.elapsed_time(b) for a, b in ev]
+
+
+def cpu_gemm_baseline(a_host, b_host, rows, n, kw, alpha):
+    """reference mm_tnn on one core (its protocol pins the process to core 0, Makefile:21);
+    falls back to the plain-C port when the compiled reference is absent"""
+    from oracle import ftnn_oracle as O
+    try:
+        os.sched_setaffinity(0, {sorted(os.sched_getaffinity(0))[0]})
+    except (AttributeError, OSError):
+        pass
+    if O.Reference.available():
+        ref, kind = O.Reference(), "reference"
+        t0 = time.perf_counter()
+        y = ref.mm(O.TNN, a_host, b_host, rows, 1, 1, n, kw, alpha)
+        dt = time.perf_counter() - t0
+    else:
+        orc, kind = O.Oracle(), "port"
+        t0 = time.perf_counter()
+        y = orc.mm(O.TNN, a_host, b_host, rows, 1, 1, n, kw, alpha)
+        dt = time.perf_counter() - t0
+    return y, dt, kind
+
+
+def conv_latency(torch, lib, typ, shape, batch, seed, reps=20):
+    """kernel-only (device buffers, HIP events) and ABI-inclusive (host pointers) latency"""
+    import numpy as np
+    from fastertnn_amd import act_is_ternary, weight_is_ternary
+    c, ih, iw, kn, kw, kh, pad, stride = shape
+    at, wt = act_is_ternary(typ), weight_is_ternary(typ)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    x = torch.randn((batch, c, ih, iw), generator=g, device="cuda")
+    thr = torch.full((batch,), 0.5 if at else 0.0, device="cuda")
+    if wt:
+        w = torch.randint(-1, 2, (kn, c, kh, kw), generator=g, device="cuda", dtype=torch.int8).float()
+    else:
+        w = torch.randint(0, 2, (kn, c, kh, kw), generator=g, device="cuda", dtype=torch.int8).float() * 2 - 1
+    wthr = torch.full((kn,), 0.5 if wt else 0.0, device="cuda")
+    qw = lib.pack_weights(w, wthr, wt)
+    oh, ow = lib.out_dim(ih, pad, kh, stride), lib.out_dim(iw, pad, kw, stride)
+    rows = torch.empty(batch * oh * ow * lib.row_words(c, kh, kw, at), dtype=torch.int64, device="cuda")
+    scratch = torch.empty(lib.pack_scratch_bytes(batch, c, ih, iw, at), dtype=torch.uint8, device="cuda")
+    y = torch.empty((batch, kn, oh, ow), device="cuda")
+
+    def step():
+        lib.conv(typ, x, thr, qw, kn, kh, kw, pad, stride, 0.5, rows=rows, scratch=scratch, out=y)
+
+    for _ in range(3):
+        step()
+    kernel_ms = sorted(event_times(torch, step, reps))[reps // 2]
+    xh, thrh, qwh = x.cpu().numpy(), thr.cpu().numpy(), qw.cpu().numpy()
+    lib.host_conv(typ, xh, thrh, qwh, kn, kh, kw, pad, stride, 0.5)
+    t = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        yh = lib.host_conv(typ, xh, thrh, qwh, kn, kh, kw, pad, stride, 0.5)
+        t.append((time.perf_counter() - t0) * 1e3)
+    out = {"kernel_ms": round(kernel_ms, 4), "abi_ms": round(sorted(t)[2], 3),
+           "gmacs_kernel": round(batch * oh * ow * kn * c * kh * kw / kernel_ms / 1e6, 1)}
+    # the reference's layer on one host core, same inputs
+    from oracle import ftnn_oracle as O
+    if O.Reference.available():
+        ref = O.Reference()
+        ref.conv(typ, xh, thrh, qwh, kn, kh, kw, pad, stride, 0.5)
+        t0 = time.perf_counter()
+        yr = ref.conv(typ, xh, thrh, qwh, kn, kh, kw, pad, stride, 0.5)
+        out["cpu_ms"] = round((time.perf_counter() - t0) * 1e3, 2)
+        out["bit_exact_vs_reference"] = bool(np.ascontiguousarray(yh).tobytes() == yr.tobytes())
+    return out
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported "
+                 "(the path shards over output rows with no exchange, see DESIGN.md)" % args.gpus)
+    import numpy as np
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    import fastertnn_amd.lib as lib
+    from fastertnn_amd import TNN, TBN, BTN
+
+    m, n, k = args.m, args.n, args.k
+    assert k % 256 == 0
+    kw = k // 64
+    alpha = 0.5
+    a = ternary_operand(torch, lib, m, k, seed=5)
+    b = ternary_operand(torch, lib, n, k, seed=6)
+    y = torch.empty((m, n, 1, 1), dtype=torch.float32, device="cuda")
+
+    def step():
+        lib.mm(TNN, a, b, m, 1, 1, n, kw, alpha, out=y)
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 26, dtype=torch.float32, device="cuda").fill_(1.0)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    macs = float(m) * n * k
+
+    # roofline of the GEMM kernel from per-launch HIP events
+    launch_ms = event_times(torch, step, max(args.steps, 5))
+    avg_ms = sum(launch_ms) / len(launch_ms)
+    valu_ops = 4.0 * m * n * (2 * kw)  # 4 vector ops per pair of 32-lane dwords, 2*kw dwords per plane
+    achieved = valu_ops / (avg_ms * 1e-3) / 1e12
+    roofline = {"bound": "valu", "achieved": round(achieved, 3), "peak": round(VALU_PEAK_TOPS, 3),
+                "unit": "Tlaneop/s", "frac": round(achieved / VALU_PEAK_TOPS, 4), "traffic": None,
+                "kernel": "k_mm<TNN>", "avg_launch_ms": round(avg_ms, 4),
+                "popcount_frac": round(achieved / 2 / VALU_PEAK_TOPS, 4),
+                "note": "peak = 256 CU x 4 SIMD x 16 lanes x 2.4 GHz int32 VALU lane-ops; "
+                        "algorithmic ops = 4 per dword pair (v_or, v_bitop3, 2 x v_bcnt)"}
+
+    cpu = None
+    if args.cpu_rows > 0:
+        rows = min(args.cpu_rows, m)
+        a_host = a[:rows * 2 * kw].cpu().numpy()
+        b_host = b.cpu().numpy()
+        from oracle.ftnn_oracle import aligned_copy
+        y_cpu, dt, kind = cpu_gemm_baseline(aligned_copy(a_host), aligned_copy(b_host), rows, n, kw, alpha)
+        y_gpu = y.view(m, n)[:rows].cpu().numpy()
+        cpu = {"value": round(float(rows) * n * k / dt / 1e9, 2), "unit": "GMAC/s", "cores": 1, "kind": kind,
+               "sample": "first %d of %d rows of A against all %d columns, K=%d (%.1f s on one core)"
+                         % (rows, m, n, k, dt),
+               "gpu_rows_bit_exact": bool(y_gpu.tobytes() == np.ascontiguousarray(y_cpu).tobytes())}
+
+    extra = None
+    if not args.no_extra:
+        extra = {
+            "tnn_conv_b1_c256_56x56_k3": conv_latency(torch, lib, TNN, (256, 56, 56, 256, 3, 3, 1, 1), 1, 2),
+            "tbn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, TBN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 3),
+            "btn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, BTN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 4),
+        }
+
+    line = {
+        "metric": "TNN GEMM ternary GMAC/s", "value": round(macs / (ms_per_step * 1e-3) / 1e9, 1),
+        "unit": "GMAC/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u32", "data": "synthetic",
+        "config": {"workload": "TNN GEMM M=%d N=%d K=%d, uniform ternary, Packing 2, PReLU 0.5 fused" % (m, n, k),
+                   "m": m, "n": n, "k": k},
+        "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

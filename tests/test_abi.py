@@ -1,0 +1,107 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol that include/ftnn.h
+declares, keeps the reference's struct layouts, and rejects bad arguments before any
+device work.  Also pins the seeded input generators.  CPU only."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "ftnn.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    return sorted(set(re.findall(r"^FTNN_API [^;(]*?\**\s*\*?(\w+)\(", text, flags=re.M)))
+
+
+def test_header_declares_the_reference_entry_points():
+    names = declared_symbols()
+    for want in ("tnns_conv", "tnns_gemm", "t2r_p2_opt", "b2r", "mm_tnn", "mm_tbn", "mm_btn", "mm_bnn"):
+        assert want in names
+    assert len(names) >= 18
+
+
+def test_library_exports_every_declared_symbol():
+    import fastertnn_amd.lib as lib
+    dll = C.CDLL(lib.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(dll, name), "libftnn_hip.so does not export " + name
+    assert sorted(lib.EXPORTS) == declared_symbols()
+
+
+def test_struct_layout_matches_the_reference(tmp_path):
+    """testcase_t is 112 bytes with `output` at 104, testcase_tnns_gemm_t 88 bytes with
+    `output` at 80 (include/tnns/data.h:4-41 on LP64)"""
+    src = tmp_path / "layout.c"
+    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "ftnn.h"\n'
+                   "int main(void){printf(\"%zu %zu %zu %zu %zu %zu %d\\n\", sizeof(testcase_t),"
+                   "offsetof(testcase_t, preluAlpha), offsetof(testcase_t, input_thresholds),"
+                   "offsetof(testcase_t, output), sizeof(testcase_tnns_gemm_t),"
+                   "offsetof(testcase_tnns_gemm_t, output), (int)BNN);return 0;}\n")
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)],
+                   check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    assert out == ["112", "48", "56", "104", "88", "80", "3"]
+    import fastertnn_amd.lib as lib
+    assert C.sizeof(lib.Testcase) == 112 and C.sizeof(lib.TestcaseGemm) == 88
+    assert lib.Testcase.output.offset == 104 and lib.TestcaseGemm.output.offset == 80
+
+
+def test_shape_helpers_match_the_oracle(oracle):
+    import fastertnn_amd.lib as lib
+    for c in (1, 3, 63, 64, 65, 127, 128, 257, 1024):
+        for (kh, kw) in ((1, 1), (3, 3), (5, 3), (7, 7)):
+            for tern in (0, 1):
+                assert lib.row_words(c, kh, kw, tern) == oracle.row_words(c, kh, kw, tern)
+    assert lib.out_dim(224, 3, 7, 2) == 112 and lib.out_dim(14, 1, 5, 2) == 6 and lib.out_dim(1, 0, 1, 1) == 1
+    assert lib.pack_scratch_bytes(2, 65, 3, 5, 1) == 2 * 15 * 2 * 16
+    assert lib.pack_scratch_bytes(2, 65, 3, 5, 0) == 2 * 15 * 2 * 8
+
+
+def test_bad_arguments_are_rejected_without_touching_the_device():
+    import fastertnn_amd.lib as lib
+    L = lib._L
+    buf = (C.c_char * 4096)()
+    p = C.addressof(buf) & ~15
+    assert L.ftnn_pack_gemm_operand(p, 4, 100, p, None) == -1          # J % 256 != 0 (src/utils.c:258)
+    assert b"256" in L.ftnn_last_error()
+    assert L.ftnn_pack_gemm_operand(None, 4, 256, p, None) == -1
+    assert L.ftnn_mm(7, p, p, 1, 1, 1, 1, 4, 0, 0.5, p, None) == -1         # unknown type
+    assert L.ftnn_mm(0, p, p, 0, 1, 1, 1, 4, 0, 0.5, p, None) == -1         # empty batch
+    assert L.ftnn_mm(0, p + 8, p, 1, 1, 1, 1, 4, 0, 0.5, p, None) == -1     # misaligned operand
+    assert L.ftnn_mm(0, None, p, 1, 1, 1, 1, 4, 0, 0.5, p, None) == -1
+    # kernel larger than the padded input
+    assert L.ftnn_quantize_im2row(1, p, p, 1, 8, 2, 2, 0, 0, 3, 3, 1, 1, p, p, None) == -1
+    assert L.ftnn_quantize_im2row(1, p, p, 1, 8, 4, 4, 0, 0, 3, 3, 0, 1, p, p, None) == -1  # stride 0
+    assert L.ftnn_conv(9, p, p, p, 1, 8, 4, 4, 4, 3, 3, 1, 1, 1, 1, 0.5, p, p, p, None) == -1
+    assert L.ftnn_pack_weights(1, p, p, 0, 8, 3, 3, p, None) == -1
+
+
+def test_missing_library_is_an_import_error(tmp_path):
+    """no silent CPU fallback: the binding refuses to import without the built library"""
+    pkg = tmp_path / "fastertnn_amd"
+    pkg.mkdir()
+    for f in ("__init__.py", "lib.py"):
+        (pkg / f).write_text(open(os.path.join(ROOT, "fastertnn_amd", f)).read())
+    r = subprocess.run(["python3", "-c", "import fastertnn_amd.lib"], cwd=str(tmp_path), capture_output=True,
+                       text=True, env={**os.environ, "PYTHONPATH": str(tmp_path)})
+    assert r.returncode != 0 and "no CPU fallback" in r.stderr
+
+
+def test_seeded_generators_are_pinned():
+    from fastertnn_amd import synth
+    z = synth.splitmix64(0, 3)
+    # SplitMix64 reference outputs for seed 0 (first three of the published test vector)
+    assert [int(v) for v in z] == [0xE220A8397B1DCDAF, 0x6E789E6AA1B965F4, 0x06C45D188009454F]
+    t = synth.ternary(1, (4096,))
+    assert set(np.unique(t)) == {-1.0, 0.0, 1.0} and abs(float(t.mean())) < 0.05
+    b = synth.binary(1, (4096,))
+    assert set(np.unique(b)) == {-1.0, 1.0}
+    g = synth.normal(1, (1 << 16,))
+    assert abs(float(g.mean())) < 0.02 and abs(float(g.std()) - 1.0) < 0.02
+    assert np.array_equal(synth.normal(9, (1000,))[100:200], synth.normal(9, (200,))[100:200])

@@ -1,0 +1,63 @@
+"""The reference's host-memory entry points (t2r_p2_opt, b2r, mm_*, tnns_conv) through the
+C ABI: results bit-exact against the oracle, returned buffers are caller-owned heap memory,
+repeated calls with changing shapes reuse the library's device workspace correctly."""
+import numpy as np
+import pytest
+
+from fastertnn_amd import TNN, TBN, BTN, BNN, TYPE_NAMES, act_is_ternary, weight_is_ternary
+from tests.cases import ALL_TYPES, EXTRA_SHAPES, REF_TEST_SHAPES, make_layer
+
+pytestmark = pytest.mark.gpu
+
+# shapes in an order that grows, shrinks and grows the workspace again
+ORDER = [6, 0, 11, 2, 10, 9, 5]
+
+
+@pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
+def test_host_entry_points(hip, oracle, typ):
+    at, wt = act_is_ternary(typ), weight_is_ternary(typ)
+    for si in ORDER:
+        shape = REF_TEST_SHAPES[si]
+        print("case", TYPE_NAMES[typ], shape, flush=True)
+        L = make_layer(typ, shape, 4, seed=2000 + si)
+        qw = oracle.pack_weights(L["w"], L["wthr"], wt)
+        rows_o = oracle.quantize_im2row(L["x"], L["thr"], L["kh"], L["kw"], L["pad"], L["stride"], at)
+        rows_h = hip.host_quantize_im2row(L["x"], L["thr"], L["kh"], L["kw"], L["pad"], L["stride"], at)
+        assert np.array_equal(rows_h, rows_o)
+        oh = hip.out_dim(L["ih"], L["pad"], L["kh"], L["stride"])
+        ow = hip.out_dim(L["iw"], L["pad"], L["kw"], L["stride"])
+        k, ku = ((L["c"] + 63) // 64) * L["kh"] * L["kw"], L["c"] * L["kh"] * L["kw"]
+        y_o = oracle.mm(typ, rows_o, qw, 4, oh, ow, L["kn"], k, L["alpha"], ku)
+        y_h = hip.host_mm(typ, rows_o, qw, 4, oh, ow, L["kn"], k, L["alpha"], ku)
+        assert y_h.tobytes() == y_o.tobytes()
+        y_c = hip.host_conv(typ, L["x"], L["thr"], qw, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], L["alpha"])
+        assert y_c.tobytes() == y_o.tobytes()
+
+
+def test_e2e_chaining_like_the_reference_driver(hip, oracle):
+    """src/timing_layers.c:189-201: the output of one tnns_conv is the next layer's input"""
+    shapes = [(64, 16, 16, 64, 3, 3, 1, 1), (64, 16, 16, 128, 1, 1, 0, 2), (128, 8, 8, 128, 3, 3, 1, 1),
+              (128, 8, 8, 10, 1, 1, 0, 1)]
+    L0 = make_layer(TNN, shapes[0], 8, seed=31)
+    thr = np.full(8, 0.5, np.float32)
+    xh, xo = L0["x"], L0["x"]
+    for i, shape in enumerate(shapes):
+        c, ih, iw, kn, kw, kh, pad, stride = shape
+        Lw = make_layer(TNN, shape, 1, seed=40 + i)
+        qw = oracle.pack_weights(Lw["w"], Lw["wthr"], True)
+        xh = hip.host_conv(TNN, xh, thr, qw, kn, kh, kw, pad, stride, 0.5)
+        xo = oracle.conv(TNN, xo, thr, qw, kn, kh, kw, pad, stride, 0.5)
+        assert xh.tobytes() == xo.tobytes(), "layer %d" % i
+
+
+def test_negative_alpha_and_alpha_one(hip, oracle):
+    """the two PReLU forms (f<=0 -> f*=alpha for TNN, r>=0 ? r : alpha*r otherwise) differ only
+    in the sign of zero for alpha < 0; both must follow the reference's form"""
+    for typ in ALL_TYPES:
+        at, wt = act_is_ternary(typ), weight_is_ternary(typ)
+        L = make_layer(typ, REF_TEST_SHAPES[1], 2, seed=77)
+        qw = oracle.pack_weights(L["w"], L["wthr"], wt)
+        for alpha in (1.0, -0.25, 0.0):
+            want = oracle.conv(typ, L["x"], L["thr"], qw, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], alpha)
+            got = hip.host_conv(typ, L["x"], L["thr"], qw, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], alpha)
+            assert got.tobytes() == want.tobytes(), (TYPE_NAMES[typ], alpha)
