@@ -12,12 +12,16 @@
 //   * lanes run along the rows of A (= output pixels, the contiguous direction
 //     of the NCHW result); each lane owns TM rows and TN columns of accumulators;
 //   * the B operand (weights) of a wavefront is wave-uniform, so it is read with
-//     scalar loads into SGPRs and enters every vector op as its one scalar
-//     source: no LDS traffic, no VGPRs and no vector instructions for B;
-//   * A tiles are copied global -> LDS with coalesced 16-byte loads, then each
-//     lane reads its own rows back with 128-bit LDS reads; the row stride is
-//     padded by 4 dwords so that the 8 lanes of a 128-byte LDS beat hit distinct
-//     banks.
+//     scalar loads (one s_load_dwordx16 per column and group) into SGPRs and
+//     enters every vector op as its one scalar source: no LDS traffic, no VGPRs
+//     and no vector instructions for B.  The load of column b+1 is issued before
+//     the arithmetic of column b;
+//   * A tiles are copied global -> registers -> LDS with coalesced 16-byte loads
+//     (the loads of chunk c+1 are issued before the arithmetic of chunk c and
+//     land in the other half of a double-buffered LDS tile: one barrier per
+//     chunk); each lane reads its own rows back with 128-bit LDS reads; the row
+//     stride is padded by 4 dwords so that the 8 lanes of a 128-byte LDS beat hit
+//     distinct banks.
 // A workgroup is 4 wavefronts sharing one A tile of 64*TM rows; wavefront w
 // computes columns [w*TN, (w+1)*TN) of the workgroup's 4*TN columns.
 #include "ftnn_internal.h"
@@ -26,7 +30,8 @@ namespace ftnn {
 
 namespace {
 
-// acc += popcount(x): one v_bcnt_u32_b32 (popcount with accumulate)
+// acc += popcount(x): one v_bcnt_u32_b32 (popcount with accumulate).  Inline asm keeps
+// the compiler from splitting the accumulation chain into partial sums plus adds.
 __device__ __forceinline__ void bcnt_acc(uint32_t& acc, uint32_t x) {
     asm("v_bcnt_u32_b32 %0, %1, %0" : "+v"(acc) : "v"(x));
 }
@@ -39,6 +44,56 @@ struct Traits {
     static constexpr int kBGroup = kBTern ? 16 : 8;
 };
 
+// one group of a B row: 8 sign dwords (s0, s1) and, for ternary B, 8 zero dwords (z0, z1)
+struct BGroup {
+    uint4 s0, s1, z0, z1;
+};
+
+template <bool TERN>
+__device__ __forceinline__ BGroup load_b(const uint32_t* bp) {
+    const uint4* q = reinterpret_cast<const uint4*>(bp);
+    BGroup r;
+    r.s0 = q[0];
+    r.s1 = q[1];
+    if (TERN) {
+        r.z0 = q[2];
+        r.z1 = q[3];
+    } else {
+        r.z0 = r.z1 = make_uint4(0, 0, 0, 0);
+    }
+    return r;
+}
+
+// the arithmetic of one dword pair; SA/ZA are per-lane (VGPR), SB/ZB wave-uniform (SGPR)
+template <int MODE>
+__device__ __forceinline__ void step(uint32_t sa, uint32_t za, uint32_t sb, uint32_t zb, uint32_t& cz,
+                                     uint32_t& cn) {
+    if (MODE == kTNN) {
+        const uint32_t z = za | zb;
+        bcnt_acc(cz, z);
+        bcnt_acc(cn, (sa ^ sb) & ~z);
+    } else if (MODE == kTBN) {
+        bcnt_acc(cn, (sa ^ sb) & ~za);
+    } else if (MODE == kBTN) {
+        bcnt_acc(cn, (sa ^ sb) & ~zb);
+    } else {
+        bcnt_acc(cn, sa ^ sb);
+    }
+}
+
+template <int MODE>
+__device__ __forceinline__ void step4(const uint4& sa, const uint4& za, const uint4& sb, const uint4& zb,
+                                      uint32_t& cz, uint32_t& cn) {
+    step<MODE>(sa.x, za.x, sb.x, zb.x, cz, cn);
+    step<MODE>(sa.y, za.y, sb.y, zb.y, cz, cn);
+    step<MODE>(sa.z, za.z, sb.z, zb.z, cz, cn);
+    step<MODE>(sa.w, za.w, sb.w, zb.w, cz, cn);
+}
+
+__device__ __forceinline__ uint32_t popc4(const uint4& v) {
+    return __popc(v.x) + __popc(v.y) + __popc(v.z) + __popc(v.w);
+}
+
 template <int MODE, int TM, int TN, int GC>
 __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
                                             const uint32_t* __restrict__ B,
@@ -47,9 +102,13 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
     using T = Traits<MODE>;
     constexpr int BM = 64 * TM;
     constexpr int AG = T::kAGroup, BG = T::kBGroup;
-    constexpr int QPG = AG / 4;          // 16-byte quads of A per group
-    constexpr int LDW = GC * AG + 4;     // LDS row stride in dwords (padded)
-    __shared__ uint32_t lds[BM * LDW];
+    constexpr int LDW = GC * AG + 4;           // LDS row stride in dwords (padded)
+    constexpr int QPR = GC * AG / 4;           // 16-byte quads per row and chunk
+    constexpr int QUADS = BM * QPR;            // quads per chunk
+    constexpr int IT = (QUADS + 255) / 256;    // staging passes per thread
+    constexpr int RPI = 256 / QPR;             // rows covered by one staging pass
+    static_assert(256 % QPR == 0, "a staging pass must cover whole rows");
+    __shared__ uint32_t lds[2][BM * LDW];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -57,10 +116,10 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
     const int col0 = (blockIdx.y * 4 + wave) * TN;
     const size_t RDA = (size_t)G * AG, RDB = (size_t)G * BG;
 
-    uint32_t cn[TM][TN];                 // popcount of "negative product" lanes
-    uint32_t cz[TM][TN];                 // TNN only: popcount of "zero product" lanes
-    uint32_t rowz[TM];                   // TBN only: popcount of za per row
-    uint32_t colz[TN];                   // BTN only: popcount of zb per column (uniform)
+    uint32_t cn[TM][TN];  // popcount of "negative product" lanes
+    uint32_t cz[TM][TN];  // TNN only: popcount of "zero product" lanes
+    uint32_t rowz[TM];    // TBN only: popcount of za per row
+    uint32_t colz[TN];    // BTN only: popcount of zb per column (wave-uniform, scalar ALU)
 #pragma unroll
     for (int a = 0; a < TM; a++) {
         rowz[a] = 0;
@@ -73,69 +132,97 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
 #pragma unroll
     for (int b = 0; b < TN; b++) colz[b] = 0;
 
-    for (int g0 = 0; g0 < G; g0 += GC) {
-        const int gc = min(GC, G - g0);
-        __syncthreads();
-        for (int e = tid; e < BM * GC * QPG; e += 256) {
-            const int r = e / (GC * QPG), q = e % (GC * QPG);
-            if (q < gc * QPG) {
-                const int64_t gr = min(row0 + r, (int64_t)M - 1);
-                const uint4 v = *reinterpret_cast<const uint4*>(A + gr * RDA + (size_t)g0 * AG + q * 4);
-                *reinterpret_cast<uint4*>(lds + r * LDW + q * 4) = v;
-            }
-        }
-        __syncthreads();
-        for (int g = 0; g < gc; g++) {
+    // columns past KN and rows past M are clamped for the loads and skipped at the store
+    const uint32_t* bcol[TN];
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
-                uint4 sa[TM], za[TM];
+    for (int b = 0; b < TN; b++) bcol[b] = B + (size_t)min(col0 + b, KN - 1) * RDB;
+
+    // staging map: pass `it` of this thread moves quad sq of tile row sr + it*RPI
+    const int sq = tid % QPR, sr = tid / QPR;
+    const bool stager = (QUADS % 256 == 0) || (tid < QUADS);
+    const uint32_t* ap[IT];
+#pragma unroll
+    for (int it = 0; it < IT; it++)
+        ap[it] = A + (size_t)min(row0 + sr + it * RPI, (int64_t)M - 1) * RDA + sq * 4;
+    uint32_t* const lw = &lds[0][0] + sr * LDW + sq * 4;
+    uint4 stage[IT];
+
+    const int nchunk = (G + GC - 1) / GC;
+    {
+        const bool on = stager && sq < min(GC, G) * (AG / 4);
+#pragma unroll
+        for (int it = 0; it < IT; it++)
+            stage[it] = on ? *reinterpret_cast<const uint4*>(ap[it]) : make_uint4(0, 0, 0, 0);
+        if (stager) {
+#pragma unroll
+            for (int it = 0; it < IT; it++)
+                *reinterpret_cast<uint4*>(lw + it * RPI * LDW) = stage[it];
+        }
+    }
+    __syncthreads();
+
+    for (int c = 0; c < nchunk; c++) {
+        const int g0 = c * GC;
+        const int gc = min(GC, G - g0);
+        const bool more = c + 1 < nchunk;
+        if (more) {  // issue the global loads of the next chunk; they land after the arithmetic
+            const bool on = stager && sq < min(GC, G - g0 - GC) * (AG / 4);
+#pragma unroll
+            for (int it = 0; it < IT; it++)
+                stage[it] = on ? *reinterpret_cast<const uint4*>(ap[it] + (size_t)(g0 + GC) * AG)
+                               : make_uint4(0, 0, 0, 0);
+        }
+        const uint32_t* lr = &lds[c & 1][0];
+        for (int g = 0; g < gc; g++) {
+            uint4 sa0[TM], sa1[TM], za0[TM], za1[TM];
+#pragma unroll
+            for (int a = 0; a < TM; a++) {
+                const uint4* lp = reinterpret_cast<const uint4*>(lr + (lane + 64 * a) * LDW + g * AG);
+                sa0[a] = lp[0];
+                sa1[a] = lp[1];
+                if (T::kATern) {
+                    za0[a] = lp[2];
+                    za1[a] = lp[3];
+                } else {
+                    za0[a] = za1[a] = make_uint4(0, 0, 0, 0);
+                }
+            }
+            if (MODE == kTBN) {  // per-row zero count, src/tnns/mm_p2_final_tbn_avx2.c:44-52
 #pragma unroll
                 for (int a = 0; a < TM; a++) {
-                    const uint32_t* lp = lds + (lane + 64 * a) * LDW + g * AG + h * 4;
-                    sa[a] = *reinterpret_cast<const uint4*>(lp);
-                    if (T::kATern) za[a] = *reinterpret_cast<const uint4*>(lp + 8);
-                }
-                if (MODE == kTBN) {
-#pragma unroll
-                    for (int a = 0; a < TM; a++) {
-                        bcnt_acc(rowz[a], za[a].x);
-                        bcnt_acc(rowz[a], za[a].y);
-                        bcnt_acc(rowz[a], za[a].z);
-                        bcnt_acc(rowz[a], za[a].w);
-                    }
-                }
-#pragma unroll
-                for (int b = 0; b < TN; b++) {
-                    const int col = min(col0 + b, KN - 1);
-                    const uint32_t* bp = B + (size_t)col * RDB + (size_t)(g0 + g) * BG + h * 4;
-                    const uint4 sb = *reinterpret_cast<const uint4*>(bp);
-                    uint4 zb = make_uint4(0, 0, 0, 0);
-                    if (T::kBTern) zb = *reinterpret_cast<const uint4*>(bp + 8);
-                    if (MODE == kBTN) colz[b] += __popc(zb.x) + __popc(zb.y) + __popc(zb.z) + __popc(zb.w);
-#pragma unroll
-                    for (int a = 0; a < TM; a++) {
-#define FTNN_STEP(c)                                                            \
-    if (MODE == kTNN) {                                                         \
-        const uint32_t z = za[a].c | zb.c;                                      \
-        const uint32_t n = (sa[a].c ^ sb.c) & ~z;                               \
-        bcnt_acc(cz[a][b], z);                                                  \
-        bcnt_acc(cn[a][b], n);                                                  \
-    } else if (MODE == kTBN) {                                                  \
-        bcnt_acc(cn[a][b], (sa[a].c ^ sb.c) & ~za[a].c);                        \
-    } else if (MODE == kBTN) {                                                  \
-        bcnt_acc(cn[a][b], (sa[a].c ^ sb.c) & ~zb.c);                           \
-    } else {                                                                    \
-        bcnt_acc(cn[a][b], sa[a].c ^ sb.c);                                     \
-    }
-                        FTNN_STEP(x)
-                        FTNN_STEP(y)
-                        FTNN_STEP(z)
-                        FTNN_STEP(w)
-#undef FTNN_STEP
-                    }
+                    bcnt_acc(rowz[a], za0[a].x);
+                    bcnt_acc(rowz[a], za0[a].y);
+                    bcnt_acc(rowz[a], za0[a].z);
+                    bcnt_acc(rowz[a], za0[a].w);
+                    bcnt_acc(rowz[a], za1[a].x);
+                    bcnt_acc(rowz[a], za1[a].y);
+                    bcnt_acc(rowz[a], za1[a].z);
+                    bcnt_acc(rowz[a], za1[a].w);
                 }
             }
+            const size_t goff = (size_t)(g0 + g) * BG;
+            BGroup cur = load_b<T::kBTern>(bcol[0] + goff);
+#pragma unroll
+            for (int b = 0; b < TN; b++) {
+                BGroup nxt = cur;
+                if (b + 1 < TN) nxt = load_b<T::kBTern>(bcol[b + 1] + goff);
+                // per-column zero count, src/tnns/mm_p2_final_btn_avx2.c:42-50
+                if (MODE == kBTN) colz[b] += popc4(cur.z0) + popc4(cur.z1);
+#pragma unroll
+                for (int a = 0; a < TM; a++) {
+                    step4<MODE>(sa0[a], za0[a], cur.s0, cur.z0, cz[a][b], cn[a][b]);
+                    step4<MODE>(sa1[a], za1[a], cur.s1, cur.z1, cz[a][b], cn[a][b]);
+                }
+                cur = nxt;
+            }
         }
+        if (more && stager) {
+            uint32_t* lwn = lw + ((c + 1) & 1) * (BM * LDW);
+#pragma unroll
+            for (int it = 0; it < IT; it++)
+                *reinterpret_cast<uint4*>(lwn + it * RPI * LDW) = stage[it];
+        }
+        __syncthreads();
     }
 
     const int lanes_total = G * 4 * 64;  // 64 * Kw
@@ -184,14 +271,15 @@ hipError_t launch_cfg(const uint32_t* A, const uint32_t* B, float* Y, int64_t M,
 template <int MODE>
 hipError_t launch_mode(const uint32_t* A, const uint32_t* B, float* Y, int64_t M, int KN, int OHW,
                        int G, int K_unpack, float alpha, hipStream_t st) {
-    // pick the largest row tile that still gives the 256 CUs a few workgroups each
+    // Tile choice (measured on MI355X): 128 x 32 tiles once they give each of the 256 CUs
+    // a dozen workgroups; layer-sized problems are one or two waves of workgroups, where
+    // smaller tiles finish sooner.
     auto wgs = [&](int tm, int tn) {
         return ((M + 64 * tm - 1) / (64 * tm)) * ((KN + 4 * tn - 1) / (4 * tn));
     };
-    if (wgs(4, 8) >= 1024) return launch_cfg<MODE, 4, 8, 2>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, st);
-    if (wgs(2, 8) >= 512) return launch_cfg<MODE, 2, 8, 2>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, st);
-    if (wgs(1, 8) >= 256) return launch_cfg<MODE, 1, 8, 2>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, st);
-    return launch_cfg<MODE, 1, 4, 2>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, st);
+    if (wgs(2, 8) >= 3072) return launch_cfg<MODE, 2, 8, 1>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, st);
+    if (wgs(1, 4) >= 2048) return launch_cfg<MODE, 1, 4, 1>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, st);
+    return launch_cfg<MODE, 1, 2, 1>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, st);
 }
 
 }  // namespace
