@@ -145,7 +145,10 @@ static float* host_mm(int type, int64_t* a, int64_t* b, int N, int OH, int OW, i
     int64_t* d_b = (int64_t*)upload(SLOT_W, b, (size_t)KN * b_words * sizeof(int64_t));
     const size_t y_bytes = M * KN * sizeof(float);
     float* d_y = (float*)dev_buf(SLOT_Y, y_bytes);
-    if (ftnn_mm(type, d_a, d_b, N, OH, OW, KN, K, K_unpack, alpha, d_y, host_stream()) != FTNN_OK)
+    const int64_t scr = ftnn_mm_scratch_bytes(FTNN_ENGINE_AUTO, type, N, OH, OW, KN, K);
+    void* d_scr = scr > 0 ? dev_buf(SLOT_SCRATCH, (size_t)scr) : nullptr;
+    if (ftnn_mm_engine(FTNN_ENGINE_AUTO, type, d_a, d_b, N, OH, OW, KN, K, K_unpack, alpha, d_y, d_scr, scr,
+                       host_stream()) != FTNN_OK)
         die("mm");
     float* y = (float*)host_alloc(y_bytes, false);
     download(y, d_y, y_bytes);
@@ -202,6 +205,63 @@ int ftnn_mm(int type, const int64_t* d_a, const int64_t* d_b, int N, int OH, int
     hipError_t e = launch_mm(type, d_a, d_b, M, OH * OW, KN, round4(K), K_unpack, prelu_alpha, d_y,
                              (hipStream_t)stream);
     return e == hipSuccess ? FTNN_OK : hip_fail(e, "mm launch");
+}
+
+// Engine choice by shape, from measurements on MI355X: the matrix-core path works on 256 x 256
+// tiles and pays two expansion passes, so it needs a few hundred tiles of real work to win.
+static int select_engine(int type, int64_t M, int KN, int Kw) {
+    (void)type;
+    const int64_t tiles = ((M + 255) / 256) * ((KN + 255) / 256);
+    if (tiles >= 128 && KN >= 256 && Kw >= 16 && 64LL * Kw < (1LL << 24)) return FTNN_ENGINE_MFMA_F4;
+    return FTNN_ENGINE_VALU;
+}
+
+int ftnn_select_engine(int type, int N, int OH, int OW, int KN, int K) {
+    if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0) return FTNN_ENGINE_VALU;
+    return select_engine(type, (int64_t)N * OH * OW, KN, round4(K));
+}
+
+int64_t ftnn_mm_scratch_bytes(int engine, int type, int N, int OH, int OW, int KN, int K) {
+    if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0) return 0;
+    const int64_t M = (int64_t)N * OH * OW;
+    const int Kw = round4(K);
+    if (engine == FTNN_ENGINE_AUTO) engine = select_engine(type, M, KN, Kw);
+    if (engine != FTNN_ENGINE_MFMA_I8 && engine != FTNN_ENGINE_MFMA_F4) return 0;
+    const bool f4 = engine == FTNN_ENGINE_MFMA_F4;
+    return mfma_fragment_bytes(f4, M, Kw) + mfma_fragment_bytes(f4, KN, Kw);
+}
+
+int ftnn_mm_engine(int engine, int type, const int64_t* d_a, const int64_t* d_b, int N, int OH, int OW,
+                   int KN, int K, int K_unpack, float prelu_alpha, float* d_y, void* d_scratch,
+                   int64_t scratch_bytes, void* stream) {
+    if (engine < FTNN_ENGINE_AUTO || engine > FTNN_ENGINE_MFMA_F4)
+        return fail(FTNN_EINVAL, "unknown engine %d", engine);
+    if (type < kTNN || type > kBNN) return fail(FTNN_EINVAL, "unknown network type %d", type);
+    if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0)
+        return fail(FTNN_EINVAL, "non-positive GEMM dimension");
+    const int64_t M = (int64_t)N * OH * OW;
+    const int Kw = round4(K);
+    if (engine == FTNN_ENGINE_AUTO) {
+        engine = select_engine(type, M, KN, Kw);
+        // AUTO never fails for lack of scratch: it falls back to the engine that needs none
+        if (engine != FTNN_ENGINE_VALU &&
+            (!d_scratch || scratch_bytes < ftnn_mm_scratch_bytes(engine, type, N, OH, OW, KN, K)))
+            engine = FTNN_ENGINE_VALU;
+    }
+    if (engine == FTNN_ENGINE_VALU)
+        return ftnn_mm(type, d_a, d_b, N, OH, OW, KN, K, K_unpack, prelu_alpha, d_y, stream);
+    if (!d_a || !d_b || !d_y) return fail(FTNN_EINVAL, "null device pointer");
+    if (!aligned16(d_a) || !aligned16(d_b)) return fail(FTNN_EINVAL, "GEMM operands must be 16-byte aligned");
+    if (M > 0x7fffffffLL) return fail(FTNN_EINVAL, "more than 2^31-1 output rows");
+    const bool f4 = engine == FTNN_ENGINE_MFMA_F4;
+    if (f4 && 64LL * Kw >= (1LL << 24))
+        return fail(FTNN_EINVAL, "K too long for exact fp32 accumulation; use the int8 engine");
+    const int64_t need = ftnn_mm_scratch_bytes(engine, type, N, OH, OW, KN, K);
+    if (!d_scratch || !aligned16(d_scratch) || scratch_bytes < need)
+        return fail(FTNN_EINVAL, "engine %d needs %lld bytes of 16-byte aligned scratch", engine, (long long)need);
+    hipError_t e = launch_mm_mfma(f4, type, d_a, d_b, M, OH * OW, KN, Kw, K_unpack, prelu_alpha, d_y,
+                                  d_scratch, (hipStream_t)stream);
+    return e == hipSuccess ? FTNN_OK : hip_fail(e, "mfma mm launch");
 }
 
 int ftnn_conv(int type, const float* d_x, const float* d_thr, const int64_t* d_qw, int N, int C,

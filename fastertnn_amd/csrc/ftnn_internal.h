@@ -27,4 +27,10 @@ hipError_t launch_mm(int type, const int64_t* d_a, const int64_t* d_b, int64_t M
                      int Kw /* words per plane, multiple of 4 */, int K_unpack, float alpha,
                      float* d_y, hipStream_t st);
 
+// ---- mfma_kernels.hip: matrix-core formulation (int8 or fp4 operands expanded into d_scratch) ----
+int64_t mfma_fragment_bytes(bool f4, int64_t rows, int Kw);
+hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* d_b, int64_t M, int OHW,
+                          int KN, int Kw, int K_unpack, float alpha, float* d_y, void* d_scratch,
+                          hipStream_t st);
+
 }  // namespace ftnn

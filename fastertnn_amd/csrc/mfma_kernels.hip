@@ -1,0 +1,343 @@
+// Matrix-core formulation of the same GEMMs (gfx950): the comparison path to the
+// vector-ALU popcount kernel of mm_kernels.hip, selected where it measures faster.
+//
+// Semantics are unchanged (src/tnns/mm_p2_final_{tnn,tbn,btn,bnn}_avx2.c): every
+// accumulator is the integer dot product of the decoded {-1,0,+1} / {-1,+1} lanes,
+// which is what the popcount formulas compute, so results stay bit-exact:
+//   * MFMA int8  (v_mfma_i32_32x32x32_i8): lanes become bytes 0x01 / 0x00 / 0xFF, int32
+//     accumulate;
+//   * MFMA fp4   (v_mfma_f32_32x32x64_f8f6f4, E2M1): lanes become nibbles 0x2 / 0x0 / 0xA
+//     (+1.0 / 0 / -1.0), fp32 accumulate -- exact while 64*Kw < 2^24, which the host
+//     checks.  Twice the matrix rate of int8 and half the operand bytes.
+//
+// Two kernels:
+//   k_expand  Packing-2 (or single-plane binary) rows -> "fragments": 1 KiB blocks
+//             holding 32 rows x 32 (int8) or 64 (fp4) lanes in exactly the register
+//             layout of an MFMA operand (lane l = (k half l/32, row l%32), 16 bytes).
+//             HBM-bound, one pass per operand.
+//   k_mfma    256 x 256 output tile per workgroup (4 wavefronts, 128 x 128 each, 256
+//             accumulator registers per lane).  Fragments travel global -> LDS with
+//             LDS-direct loads (no VGPRs, and a fragment lands contiguously, so the
+//             later 128-bit LDS reads are conflict-free without padding), through a
+//             4-stage ring; one barrier per step.  LDS reads of the next fragment and
+//             the DMA issue are interleaved with the MFMAs of the current one.
+#include <type_traits>
+
+#include "ftnn_internal.h"
+
+namespace ftnn {
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kKF = 2;   // fragments per row-block and step
+constexpr int kNS = 4;   // LDS ring depth
+constexpr int kFR = 16 * kKF;            // fragments per step: (8 P + 8 Q row-blocks) x kKF
+constexpr int kFW = kFR / 4;             // fragments staged by one wavefront per step
+constexpr size_t kLdsBytes = (size_t)kNS * kFR * 1024;
+
+// ------------------------------------------------------------------ expansion
+// grid (row-blocks, groups), block 256: thread = (row r = t%32, dword pair dq = t/32).
+// A group is 4 words (256 lanes) of a packed row: 16 dwords (8 sign, 8 zero) for ternary
+// rows, 8 dwords for binary rows.  Rows past `rows` expand to zeros.
+template <bool F4, bool TERN>
+__global__ __launch_bounds__(256) void k_expand(const uint32_t* __restrict__ P, int rows, int G,
+                                                uint4* __restrict__ out) {
+    const int rb = blockIdx.x, g = blockIdx.y, t = threadIdx.x;
+    const int r = t & 31, dq = t >> 5;
+    const int row = min(rb * 32 + r, rows - 1);
+    const bool live = rb * 32 + r < rows;
+    uint32_t s, nz;
+    if (TERN) {
+        const uint32_t* src = P + ((size_t)row * G + g) * 16;
+        nz = live ? ~src[8 + dq] : 0u;
+        s = src[dq] & nz;   // a lane flagged zero is zero whatever its sign bit says
+    } else {
+        const uint32_t* src = P + ((size_t)row * G + g) * 8;
+        nz = live ? 0xffffffffu : 0u;
+        s = src[dq] & nz;
+    }
+    if (F4) {
+        // fragment = one 64-lane word: dword dq&1 is its k half; nibble = sign<<3 | nonzero<<1
+        uint4* frag = out + ((size_t)rb * (G * 4) + (g * 4 + (dq >> 1))) * 64;
+        uint32_t o[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            uint32_t a = (s >> (8 * q)) & 0xffu, b = (nz >> (8 * q)) & 0xffu;
+            a = (a | (a << 12)) & 0x000F000Fu;
+            a = (a | (a << 6)) & 0x03030303u;
+            a = (a | (a << 3)) & 0x11111111u;
+            b = (b | (b << 12)) & 0x000F000Fu;
+            b = (b | (b << 6)) & 0x03030303u;
+            b = (b | (b << 3)) & 0x11111111u;
+            o[q] = (a << 3) | (b << 1);
+        }
+        frag[(dq & 1) * 32 + r] = make_uint4(o[0], o[1], o[2], o[3]);
+    } else {
+        // fragment = one 32-lane dword: its two 16-lane halves are the k halves
+        uint4* frag = out + ((size_t)rb * (G * 8) + (g * 8 + dq)) * 64;
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const uint32_t sh = (s >> (16 * half)) & 0xffffu, nh = (nz >> (16 * half)) & 0xffffu;
+            uint32_t o[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                // 4 bits -> 4 byte LSBs: bit i lands on bit 8i, no carries
+                const uint32_t sb = (((sh >> (4 * q)) & 15u) * 0x204081u) & 0x01010101u;
+                const uint32_t nb = (((nh >> (4 * q)) & 15u) * 0x204081u) & 0x01010101u;
+                o[q] = nb | (sb * 0xffu);
+            }
+            frag[half * 32 + r] = make_uint4(o[0], o[1], o[2], o[3]);
+        }
+    }
+}
+
+// ----------------------------------------------------------------------- GEMM
+template <bool F4>
+struct Acc {
+    typedef v16i type;
+};
+template <>
+struct Acc<true> {
+    typedef v16f type;
+};
+
+template <bool F4>
+__device__ __forceinline__ void mfma(typename Acc<F4>::type& c, const uint4& a, const uint4& b) {
+    if constexpr (F4) {
+        const v8i va = {(int)a.x, (int)a.y, (int)a.z, (int)a.w, 0, 0, 0, 0};
+        const v8i vb = {(int)b.x, (int)b.y, (int)b.z, (int)b.w, 0, 0, 0, 0};
+        // cbsz = blgp = 4: both operands E2M1; scale operands 0 select the unscaled instruction
+        c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va, vb, c, 4, 4, 0, 0, 0, 0);
+    } else {
+        const v4i va = {(int)a.x, (int)a.y, (int)a.z, (int)a.w};
+        const v4i vb = {(int)b.x, (int)b.y, (int)b.z, (int)b.w};
+        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(va, vb, c, 0, 0, 0);
+    }
+}
+
+// LDS-direct load of 16 bytes per lane: the 64 lanes land contiguously at lds_byte_addr.
+// Issued through inline asm so that the compiler does not order its own LDS reads against
+// it; the kernel waits for it by hand (s_waitcnt vmcnt before the barrier that publishes
+// the buffer).  M0 carries the LDS address; one wait state is required after writing M0.
+__device__ __forceinline__ void dma16(const uint4* gsrc, uint32_t lds_byte_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gsrc), "s"(lds_byte_addr)
+                 : "memory");
+}
+
+// P operand = MFMA A side (its rows index the accumulator registers), Q operand = MFMA B
+// side (its rows run along the lanes).  SWAP = false: P = activation rows i, Q = weight
+// rows j (lanes along j: contiguous for a row-major m x n result).  SWAP = true: P =
+// weights, Q = activations (lanes along i: contiguous for an NCHW result with OHW > 1).
+// The epilogue computes r = acc - bias, then PReLU in the reference's form for the type:
+// form 0 "f = r; if (f <= 0) f *= alpha" (mm_p2_final_tnn_avx2.c:204-208), form 1
+// "r >= 0 ? r : alpha * r" (mm_p2_final_tbn_avx2.c:73).
+template <bool F4, bool SWAP>
+__global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, const uint4* __restrict__ Qf,
+                                              float* __restrict__ Y, int M, int KN, int OHW, int KB,
+                                              int bias, int form, float alpha) {
+    extern __shared__ uint4 lds[];   // kNS buffers of kFR KiB
+    typedef typename Acc<F4>::type acc_t;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wy = wave >> 1, wx = wave & 1;
+    const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN;
+    const int prb0 = blockIdx.x * 8, qrb0 = blockIdx.y * 8;
+    const int prbmax = (prow + 31) / 32 - 1, qrbmax = (qrow + 31) / 32 - 1;
+    acc_t acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[a][b][e] = 0;
+
+    // fragment f of a step: side f / (8*kKF) (0 = P, 1 = Q), row-block (f / kKF) % 8, k fragment
+    // f % kKF; row-blocks past the operand are clamped (their results are never stored)
+    const uint4* src[kFW];
+#pragma unroll
+    for (int i = 0; i < kFW; i++) {
+        const int f = wave * kFW + i;
+        const int side = f / (8 * kKF), rbi = (f / kKF) % 8, kbi = f % kKF;
+        const uint4* base = side == 0 ? Pf + ((size_t)min(prb0 + rbi, prbmax) * KB + kbi) * 64
+                                      : Qf + ((size_t)min(qrb0 + rbi, qrbmax) * KB + kbi) * 64;
+        src[i] = base + lane;
+    }
+    const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)lds);
+    const int nstep = KB / kKF;
+    auto stage = [&](int step) {
+        const uint32_t dst = lds0 + (uint32_t)(step % kNS) * (kFR * 1024) + wave * (kFW * 1024);
+#pragma unroll
+        for (int i = 0; i < kFW; i++) dma16(src[i] + (size_t)step * kKF * 64, dst + i * 1024);
+    };
+    uint4 fa[2][4], fb[2][4];
+    // one LDS read of fragment k of buffer `buf` into register set `set`, in the order the MFMAs
+    // consume them: i = 0: fa0, 1..4: fb0..fb3, 5..7: fa1..fa3
+    auto ldone = [&](int buf, int k, int set, int i) {
+        const uint4* L = lds + (size_t)buf * kFR * 64;
+        if (i == 0) fa[set][0] = L[((wy * 4 + 0) * kKF + k) * 64 + lane];
+        else if (i <= 4) fb[set][i - 1] = L[((8 + wx * 4 + (i - 1)) * kKF + k) * 64 + lane];
+        else fa[set][i - 4] = L[((wy * 4 + (i - 4)) * kKF + k) * 64 + lane];
+    };
+    auto mfma2 = [&](int set, int i) {
+        mfma<F4>(acc[(2 * i) / 4][(2 * i) % 4], fa[set][(2 * i) / 4], fb[set][(2 * i) % 4]);
+        mfma<F4>(acc[(2 * i + 1) / 4][(2 * i + 1) % 4], fa[set][(2 * i + 1) / 4], fb[set][(2 * i + 1) % 4]);
+    };
+
+    // prologue: the first kNS stages in flight, wait for stage 0 only
+#pragma unroll
+    for (int p = 0; p < kNS; p++)
+        if (p < nstep) stage(p);
+    if (nstep >= kNS) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFW * (kNS - 1)) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 8; i++) ldone(0, 0, 0, i);
+
+    auto step_body = [&](int s, auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;   // FULL: s + kNS < nstep
+#pragma unroll
+        for (int k = 0; k < kKF; k++) {
+            const int set = k & 1;
+            if (k + 1 < kKF) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    ldone(s % kNS, k + 1, set ^ 1, i);
+                    mfma2(set, i);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+                // Last fragment of the step: all of this step is in registers.  Stage s+1 must
+                // have landed (stages s+2 .. s+kNS-1 may still be in flight); after the barrier
+                // buffer s % kNS is free for stage s+kNS.
+                if (FULL || s + kNS - 1 < nstep) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFW * (kNS - 2)) : "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                const bool do_ld = FULL || s + 1 < nstep;
+                const uint32_t dst = lds0 + (uint32_t)(s % kNS) * (kFR * 1024) + wave * (kFW * 1024);
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    if (FULL) {
+#pragma unroll
+                        for (int j = 0; j < kFW / 8; j++)
+                            dma16(src[i * (kFW / 8) + j] + (size_t)(s + kNS) * kKF * 64,
+                                  dst + (i * (kFW / 8) + j) * 1024);
+                    }
+                    if (do_ld) ldone((s + 1) % kNS, 0, set ^ 1, i);
+                    mfma2(set, i);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+    };
+    int s = 0;
+    for (; s + kNS < nstep; s++) step_body(s, std::true_type{});
+    for (; s < nstep; s++) step_body(s, std::false_type{});
+
+    // accumulator e of block (a, b): P row = 32*prb + 8*(e/4) + 4*(lane/32) + e%4, Q row = 32*qrb + lane%32
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const int q = (qrb0 + wx * 4 + b) * 32 + (lane & 31);
+            const int pbase = (prb0 + wy * 4 + a) * 32 + 4 * (lane >> 5);
+            size_t qoff = 0;   // SWAP: q = i is fixed per block, hoist its image split
+            if (SWAP) {
+                const int img = q / OHW;
+                qoff = (size_t)img * KN * OHW + (q - img * OHW);
+            }
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int p = pbase + 8 * (e >> 2) + (e & 3);
+                const int i = SWAP ? q : p, j = SWAP ? p : q;
+                if (i < M && j < KN) {
+                    const int r = (int)acc[a][b][e] - bias;
+                    float f;
+                    if (form == 0) {
+                        f = (float)r;
+                        if (f <= 0) f *= alpha;
+                    } else {
+                        f = r >= 0 ? (float)r : alpha * r;
+                    }
+                    size_t o;
+                    if (SWAP) {
+                        o = qoff + (size_t)j * OHW;
+                    } else if (OHW == 1) {
+                        o = (size_t)i * KN + j;
+                    } else {
+                        const int img = i / OHW;
+                        o = ((size_t)img * KN + j) * OHW + (i - img * OHW);
+                    }
+                    Y[o] = f;
+                }
+            }
+        }
+}
+
+template <bool F4, bool SWAP>
+hipError_t launch_gemm(const uint4* Pf, const uint4* Qf, float* Y, int M, int KN, int OHW, int KB,
+                       int bias, int form, float alpha, hipStream_t st) {
+    auto kern = k_mfma<F4, SWAP>;
+    static bool configured = false;   // the opt-in to more than 64 KiB of dynamic LDS is per kernel
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN;
+    dim3 grid((prow + 255) / 256, (qrow + 255) / 256);
+    if (grid.y > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(kern, grid, dim3(256), kLdsBytes, st, Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha);
+    return hipGetLastError();
+}
+
+template <bool F4>
+hipError_t launch_expand(bool tern, const uint32_t* rows_ptr, int rows, int G, uint4* out, hipStream_t st) {
+    dim3 grid((rows + 31) / 32, G);
+    if (grid.y > 65535) return hipErrorInvalidValue;
+    if (tern) hipLaunchKernelGGL((k_expand<F4, true>), grid, dim3(256), 0, st, rows_ptr, rows, G, out);
+    else hipLaunchKernelGGL((k_expand<F4, false>), grid, dim3(256), 0, st, rows_ptr, rows, G, out);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+int64_t mfma_fragment_bytes(bool f4, int64_t rows, int Kw) {
+    // 1 KiB fragments: 32 rows x one word (fp4) or half a word (int8)
+    return ((rows + 31) / 32) * (int64_t)(f4 ? Kw : 2 * Kw) * 1024;
+}
+
+hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* d_b, int64_t M, int OHW,
+                          int KN, int Kw, int K_unpack, float alpha, float* d_y, void* d_scratch,
+                          hipStream_t st) {
+    const bool a_tern = (type == kTNN || type == kTBN), b_tern = (type == kTNN || type == kBTN);
+    const int G = Kw / 4, KB = f4 ? Kw : 2 * Kw;
+    uint4* Af = static_cast<uint4*>(d_scratch);
+    uint4* Bf = reinterpret_cast<uint4*>(static_cast<char*>(d_scratch) + mfma_fragment_bytes(f4, M, Kw));
+    const uint32_t* A = reinterpret_cast<const uint32_t*>(d_a);
+    const uint32_t* B = reinterpret_cast<const uint32_t*>(d_b);
+    hipError_t e = f4 ? launch_expand<true>(a_tern, A, (int)M, G, Af, st) : launch_expand<false>(a_tern, A, (int)M, G, Af, st);
+    if (e != hipSuccess) return e;
+    e = f4 ? launch_expand<true>(b_tern, B, KN, G, Bf, st) : launch_expand<false>(b_tern, B, KN, G, Bf, st);
+    if (e != hipSuccess) return e;
+    // BNN: the lanes past K_unpack are +1 in both operands and add 64*Kw - K_unpack to the dot
+    // product; the reference's K_unpack - 2*popc(a^b) leaves them out (mm_p2_final_bnn_avx2.c:55-58)
+    const int bias = type == kBNN ? 64 * Kw - K_unpack : 0;
+    const int form = type == kTNN ? 0 : 1;
+    const bool swap = OHW > 1;
+    if (f4) {
+        return swap ? launch_gemm<true, true>(Bf, Af, d_y, (int)M, KN, OHW, KB, bias, form, alpha, st)
+                    : launch_gemm<true, false>(Af, Bf, d_y, (int)M, KN, OHW, KB, bias, form, alpha, st);
+    }
+    return swap ? launch_gemm<false, true>(Bf, Af, d_y, (int)M, KN, OHW, KB, bias, form, alpha, st)
+                : launch_gemm<false, false>(Af, Bf, d_y, (int)M, KN, OHW, KB, bias, form, alpha, st);
+}
+
+}  // namespace ftnn

@@ -31,6 +31,10 @@ _L.ftnn_row_words.restype = C.c_int64
 _L.ftnn_pack_scratch_bytes.restype = C.c_int64
 _L.ftnn_quantize_im2row.argtypes = [C.c_int, _vp, _vp] + [C.c_int] * 10 + [_vp, _vp, _vp]
 _L.ftnn_mm.argtypes = [C.c_int, _vp, _vp] + [C.c_int] * 6 + [C.c_float, _vp, _vp]
+_L.ftnn_mm_scratch_bytes.restype = C.c_int64
+_L.ftnn_mm_scratch_bytes.argtypes = [C.c_int] * 7
+_L.ftnn_select_engine.argtypes = [C.c_int] * 6
+_L.ftnn_mm_engine.argtypes = [C.c_int, C.c_int, _vp, _vp] + [C.c_int] * 6 + [C.c_float, _vp, _vp, C.c_int64, _vp]
 _L.ftnn_conv.argtypes = [C.c_int, _vp, _vp, _vp] + [C.c_int] * 11 + [C.c_float, _vp, _vp, _vp, _vp]
 _L.ftnn_pack_weights.argtypes = [C.c_int, _vp, _vp] + [C.c_int] * 4 + [_vp, _vp]
 _L.ftnn_pack_gemm_operand.argtypes = [_vp, C.c_int, C.c_int, _vp, _vp]
@@ -48,7 +52,11 @@ _L.tnns_gemm.restype = None
 EXPORTS = ("tnns_conv", "tnns_gemm", "t2r_p2_opt", "b2r", "mm_tnn", "mm_tbn", "mm_btn", "mm_bnn",
            "ftnn_last_error", "ftnn_version", "ftnn_out_dim", "ftnn_row_words",
            "ftnn_pack_scratch_bytes", "ftnn_quantize_im2row", "ftnn_mm", "ftnn_conv",
-           "ftnn_pack_weights", "ftnn_pack_gemm_operand")
+           "ftnn_pack_weights", "ftnn_pack_gemm_operand", "ftnn_select_engine", "ftnn_mm_scratch_bytes",
+           "ftnn_mm_engine")
+
+ENGINE_AUTO, ENGINE_VALU, ENGINE_MFMA_I8, ENGINE_MFMA_F4 = 0, 1, 2, 3
+ENGINE_NAMES = {ENGINE_VALU: "valu", ENGINE_MFMA_I8: "mfma_i8", ENGINE_MFMA_F4: "mfma_f4"}
 
 
 class FtnnError(RuntimeError):
@@ -116,6 +124,29 @@ def mm(typ, a, b, n, oh, ow, kn, k, alpha, k_unpack=0, out=None):
         out = torch.empty((n, kn, oh, ow), dtype=torch.float32, device=a.device)
     _check(_L.ftnn_mm(typ, _dev(a), _dev(b), n, oh, ow, kn, k, k_unpack, alpha, _dev(out, torch.float32),
                       _stream()))
+    return out
+
+
+def select_engine(typ, n, oh, ow, kn, k):
+    return int(_L.ftnn_select_engine(typ, n, oh, ow, kn, k))
+
+
+def mm_scratch_bytes(engine, typ, n, oh, ow, kn, k):
+    return int(_L.ftnn_mm_scratch_bytes(engine, typ, n, oh, ow, kn, k))
+
+
+def mm_engine(engine, typ, a, b, n, oh, ow, kn, k, alpha, k_unpack=0, out=None, scratch=None):
+    """ftnn_mm_engine: the GEMM on an explicit engine (or AUTO); scratch is allocated if not given."""
+    import torch
+    if out is None:
+        out = torch.empty((n, kn, oh, ow), dtype=torch.float32, device=a.device)
+    need = mm_scratch_bytes(engine, typ, n, oh, ow, kn, k)
+    if scratch is None and need > 0:
+        scratch = torch.empty(need, dtype=torch.uint8, device=a.device)
+    sp = _dev(scratch) if scratch is not None else None
+    sb = scratch.numel() * scratch.element_size() if scratch is not None else 0
+    _check(_L.ftnn_mm_engine(engine, typ, _dev(a), _dev(b), n, oh, ow, kn, k, k_unpack, alpha,
+                             _dev(out, torch.float32), sp, sb, _stream()))
     return out
 
 

@@ -151,6 +151,33 @@ FTNN_API int ftnn_mm(int type, const int64_t *d_a, const int64_t *d_b, int N, in
             int K, int K_unpack, float prelu_alpha, float *d_y, void *stream);
 
 /*
+ * GEMM engines.  The reference has one arithmetic (XOR/AND/popcount on bit-planes); on
+ * MI355X the same integer dot products can also run on the matrix cores after the lanes
+ * are expanded to int8 or fp4 (E2M1 holds -1, 0, +1 exactly).  All engines give the same
+ * bits.  AUTO picks per shape what measured fastest.
+ */
+#define FTNN_ENGINE_AUTO 0
+#define FTNN_ENGINE_VALU 1    /* bit-plane popcount on the vector ALU, no scratch   */
+#define FTNN_ENGINE_MFMA_I8 2 /* v_mfma_i32_32x32x32_i8 on expanded operands         */
+#define FTNN_ENGINE_MFMA_F4 3 /* v_mfma_f32_32x32x64_f8f6f4 (fp4) on expanded operands */
+
+/* the engine FTNN_ENGINE_AUTO resolves to for this shape (never AUTO) */
+FTNN_API int ftnn_select_engine(int type, int N, int OH, int OW, int KN, int K);
+
+/* device scratch, in bytes, that ftnn_mm_engine needs for `engine` (0 for the VALU engine;
+ * for AUTO the amount of the engine it resolves to) */
+FTNN_API int64_t ftnn_mm_scratch_bytes(int engine, int type, int N, int OH, int OW, int KN, int K);
+
+/*
+ * ftnn_mm with an explicit engine.  d_scratch (16-byte aligned, scratch_bytes long) holds
+ * the expanded operands of the matrix-core engines; it may be NULL for the VALU engine.
+ * No counterpart in the reference: its mm_* have a single implementation.
+ */
+FTNN_API int ftnn_mm_engine(int engine, int type, const int64_t *d_a, const int64_t *d_b, int N, int OH,
+                   int OW, int KN, int K, int K_unpack, float prelu_alpha, float *d_y,
+                   void *d_scratch, int64_t scratch_bytes, void *stream);
+
+/*
  * One conv layer on the device: ftnn_quantize_im2row then ftnn_mm
  * (src/tnns/tnns_cpu_mm_p2.c:6-80).  d_rows holds N*OH*OW packed rows.
  */

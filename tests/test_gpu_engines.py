@@ -1,0 +1,88 @@
+"""The three GEMM engines (vector-ALU popcount, MFMA int8, MFMA fp4) give the same bits as the
+oracle for all four network types, for GEMM-shaped (row-major) and conv-shaped (NCHW) outputs,
+ragged tiles and K tails."""
+import numpy as np
+import pytest
+
+from fastertnn_amd import TNN, TBN, BTN, BNN, TYPE_NAMES, act_is_ternary, weight_is_ternary
+from tests.cases import ALL_TYPES, REF_TEST_SHAPES, EXTRA_SHAPES, make_layer
+
+pytestmark = pytest.mark.gpu
+
+LAYERS = [REF_TEST_SHAPES[i] for i in (1, 5, 6, 8, 9, 10)] + [EXTRA_SHAPES[0], EXTRA_SHAPES[3],
+                                                            (64, 20, 20, 300, 3, 3, 1, 1)]
+
+
+def _dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
+@pytest.mark.parametrize("si", range(len(LAYERS)))
+def test_engines_on_layers(hip, oracle, typ, si):
+    shape = LAYERS[si]
+    batch = 3
+    L = make_layer(typ, shape, batch, seed=4000 + 13 * si + typ)
+    print("case", TYPE_NAMES[typ], shape, flush=True)
+    at, wt = act_is_ternary(typ), weight_is_ternary(typ)
+    qw = oracle.pack_weights(L["w"], L["wthr"], wt)
+    rows = oracle.quantize_im2row(L["x"], L["thr"], L["kh"], L["kw"], L["pad"], L["stride"], at)
+    oh = hip.out_dim(L["ih"], L["pad"], L["kh"], L["stride"])
+    ow = hip.out_dim(L["iw"], L["pad"], L["kw"], L["stride"])
+    k, ku = ((L["c"] + 63) // 64) * L["kh"] * L["kw"], L["c"] * L["kh"] * L["kw"]
+    for alpha in (0.5, -0.25):
+        want = oracle.mm(typ, rows, qw, batch, oh, ow, L["kn"], k, alpha, ku)
+        a_d, b_d = _dev(rows), _dev(qw)
+        for eng in (hip.ENGINE_VALU, hip.ENGINE_MFMA_I8, hip.ENGINE_MFMA_F4, hip.ENGINE_AUTO):
+            got = hip.mm_engine(eng, typ, a_d, b_d, batch, oh, ow, L["kn"], k, alpha, ku).cpu().numpy()
+            assert got.tobytes() == want.tobytes(), "engine %d alpha %g" % (eng, alpha)
+
+
+@pytest.mark.parametrize("mnp", [(300, 70, 768), (257, 513, 256), (1024, 1024, 2048), (33, 1000, 512)])
+def test_engines_on_gemm_operands(hip, oracle, mnp):
+    from fastertnn_amd import synth
+    m, n, p = mnp
+    a, b = synth.ternary(m, (m, p)), synth.ternary(n + 1, (n, p))
+    ap, bp = oracle.pack_gemm_operand(a), oracle.pack_gemm_operand(b)
+    want = oracle.mm(TNN, ap, bp, m, 1, 1, n, p // 64, 0.5)
+    assert np.array_equal(oracle.gemm(ap, bp, m, n, p // 64), a @ b.T)
+    a_d, b_d = _dev(ap), _dev(bp)
+    for eng in (hip.ENGINE_VALU, hip.ENGINE_MFMA_I8, hip.ENGINE_MFMA_F4):
+        got = hip.mm_engine(eng, TNN, a_d, b_d, m, 1, 1, n, p // 64, 0.5).cpu().numpy()
+        assert got.tobytes() == want.tobytes(), "engine %d" % eng
+
+
+def test_lanes_flagged_zero_and_negative_count_as_zero(hip, oracle):
+    """a lane with both its sign and its zero bit set is zero in the reference's formula
+    (za|zb masks it); the expanded operands must agree"""
+    rng = np.random.default_rng(3)
+    m, n, kw = 70, 40, 8
+    a = rng.integers(-2 ** 63, 2 ** 63, size=m * 2 * kw, dtype=np.int64)
+    b = rng.integers(-2 ** 63, 2 ** 63, size=n * 2 * kw, dtype=np.int64)
+    want = oracle.mm(TNN, a, b, m, 1, 1, n, kw, 0.5)
+    for eng in (hip.ENGINE_VALU, hip.ENGINE_MFMA_I8, hip.ENGINE_MFMA_F4):
+        got = hip.mm_engine(eng, TNN, _dev(a), _dev(b), m, 1, 1, n, kw, 0.5).cpu().numpy()
+        assert got.tobytes() == want.tobytes(), "engine %d" % eng
+
+
+def test_engine_argument_checks(hip):
+    import torch
+    a = torch.zeros(64 * 8, dtype=torch.int64, device="cuda")
+    y = torch.empty((8, 8, 1, 1), device="cuda")
+    L = hip._L
+    s = hip._stream()
+    assert L.ftnn_mm_engine(9, 0, a.data_ptr(), a.data_ptr(), 8, 1, 1, 8, 4, 0, 0.5, y.data_ptr(), None, 0, s) == -1
+    # an explicit matrix-core engine without scratch is an error ...
+    assert L.ftnn_mm_engine(hip.ENGINE_MFMA_F4, 0, a.data_ptr(), a.data_ptr(), 8, 1, 1, 8, 4, 0, 0.5, y.data_ptr(),
+                            None, 0, s) == -1
+    assert b"scratch" in L.ftnn_last_error()
+    # ... AUTO without scratch falls back to the engine that needs none
+    assert L.ftnn_mm_engine(hip.ENGINE_AUTO, 0, a.data_ptr(), a.data_ptr(), 8, 1, 1, 8, 4, 0, 0.5, y.data_ptr(),
+                            None, 0, s) == 0
+    torch.cuda.synchronize()
+    assert hip.mm_scratch_bytes(hip.ENGINE_VALU, 0, 8192, 1, 1, 8192, 512) == 0
+    assert hip.mm_scratch_bytes(hip.ENGINE_MFMA_F4, 0, 8192, 1, 1, 8192, 512) == 2 * 256 * 512 * 1024
+    assert hip.mm_scratch_bytes(hip.ENGINE_MFMA_I8, 0, 33, 1, 1, 1, 4) == (2 + 1) * 8 * 1024
+    assert hip.select_engine(0, 8192, 1, 1, 8192, 512) == hip.ENGINE_MFMA_F4
+    assert hip.select_engine(0, 1, 56, 56, 256, 36) == hip.ENGINE_VALU
