@@ -157,9 +157,12 @@ def main():
     a = ternary_operand(torch, lib, m, k, seed=5)
     b = ternary_operand(torch, lib, n, k, seed=6)
     y = torch.empty((m, n, 1, 1), dtype=torch.float32, device="cuda")
+    auto = lib.select_engine(TNN, m, 1, 1, n, kw)
+    scratch = torch.empty(max(lib.mm_scratch_bytes(e, TNN, m, 1, 1, n, kw) for e in lib.ENGINE_NAMES) or 16,
+                          dtype=torch.uint8, device="cuda")
 
-    def step():
-        lib.mm(TNN, a, b, m, 1, 1, n, kw, alpha, out=y)
+    def step():   # the timed hot path: packed operands in, fp32 result out, engine chosen by the library
+        lib.mm_engine(lib.ENGINE_AUTO, TNN, a, b, m, 1, 1, n, kw, alpha, out=y, scratch=scratch)
 
     if args.copy_calibration:
         src = torch.empty(1 << 26, dtype=torch.float32, device="cuda").fill_(1.0)
@@ -178,18 +181,56 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
     macs = float(m) * n * k
+    reps = max(args.steps, 5)
 
-    # roofline of the GEMM kernel from per-launch HIP events
-    launch_ms = event_times(torch, step, max(args.steps, 5))
-    avg_ms = sum(launch_ms) / len(launch_ms)
-    valu_ops = 4.0 * m * n * (2 * kw)  # 4 vector ops per pair of 32-lane dwords, 2*kw dwords per plane
-    achieved = valu_ops / (avg_ms * 1e-3) / 1e12
-    roofline = {"bound": "valu", "achieved": round(achieved, 3), "peak": round(VALU_PEAK_TOPS, 3),
-                "unit": "Tlaneop/s", "frac": round(achieved / VALU_PEAK_TOPS, 4), "traffic": None,
-                "kernel": "k_mm<TNN>", "avg_launch_ms": round(avg_ms, 4),
-                "popcount_frac": round(achieved / 2 / VALU_PEAK_TOPS, 4),
-                "note": "peak = 256 CU x 4 SIMD x 16 lanes x 2.4 GHz int32 VALU lane-ops; "
-                        "algorithmic ops = 4 per dword pair (v_or, v_bitop3, 2 x v_bcnt)"}
+    def mean(v):
+        return sum(v) / len(v)
+
+    # every engine on the same operands, per-launch HIP events; the whole call (expansion included)
+    engines = {}
+    y_ref = None
+    for eng, name in lib.ENGINE_NAMES.items():
+        def run(eng=eng):
+            lib.mm_engine(eng, TNN, a, b, m, 1, 1, n, kw, alpha, out=y, scratch=scratch)
+        run()
+        torch.cuda.synchronize()
+        if y_ref is None:
+            y_ref = y.clone()
+        same = bool(torch.equal(y, y_ref))
+        t = mean(event_times(torch, run, reps))
+        engines[name] = {"call_ms": round(t, 4), "gmacs": round(macs / t / 1e6, 1), "same_bits_as_valu": same}
+    del y_ref
+
+    # rooflines of the dominant kernels, each timed alone with HIP events on the launch stream
+    valu_ms = engines["valu"]["call_ms"]   # the VALU engine is one kernel
+    valu_ops = 4.0 * m * n * (2 * kw)      # 4 vector ops per pair of 32-lane dwords, 2*kw dwords per plane
+    valu_ach = valu_ops / (valu_ms * 1e-3) / 1e12
+    roofline_valu = {"bound": "valu", "achieved": round(valu_ach, 3), "peak": round(VALU_PEAK_TOPS, 3),
+                     "unit": "Tlaneop/s", "frac": round(valu_ach / VALU_PEAK_TOPS, 4), "traffic": None,
+                     "kernel": "k_mm<TNN,2,8,1>", "avg_launch_ms": valu_ms,
+                     "popcount_frac": round(valu_ach / 2 / VALU_PEAK_TOPS, 4),
+                     "note": "peak = 256 CU x 4 SIMD x 16 lanes x 2.4 GHz int32 VALU lane-ops; "
+                             "algorithmic ops = 4 per dword pair (v_or, v_bitop3, 2 x v_bcnt)"}
+    mfma = {}
+    for eng, kernel, peak in ((lib.ENGINE_MFMA_I8, "k_mfma<int8>", 5000.0), (lib.ENGINE_MFMA_F4, "k_mfma<fp4>", 10100.0)):
+        a_exp = lib.expand_rows(eng, a, m, kw, True)
+        b_exp = lib.expand_rows(eng, b, n, kw, True)
+
+        def gemm(eng=eng, a_exp=a_exp, b_exp=b_exp):
+            lib.mm_expanded(eng, TNN, a_exp, b_exp, m, 1, 1, n, kw, alpha, out=y)
+
+        def expand(eng=eng, a_exp=a_exp):
+            lib.expand_rows(eng, a, m, kw, True, out=a_exp)
+        gemm()
+        t = mean(event_times(torch, gemm, reps))
+        te = mean(event_times(torch, expand, reps))
+        ach = 2.0 * macs / (t * 1e-3) / 1e12
+        mfma[eng] = {"bound": "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "TOP/s" if eng == lib.ENGINE_MFMA_I8 else "TFLOP/s",
+                     "frac": round(ach / peak, 4), "traffic": None, "kernel": kernel, "avg_launch_ms": round(t, 4),
+                     "expand_one_operand_ms": round(te, 4)}
+        del a_exp, b_exp
+    roofline = {lib.ENGINE_VALU: roofline_valu, lib.ENGINE_MFMA_I8: mfma[lib.ENGINE_MFMA_I8],
+                lib.ENGINE_MFMA_F4: mfma[lib.ENGINE_MFMA_F4]}[auto]
 
     cpu = None
     if args.cpu_rows > 0:
@@ -216,10 +257,13 @@ def main():
         "metric": "TNN GEMM ternary GMAC/s", "value": round(macs / (ms_per_step * 1e-3) / 1e9, 1),
         "unit": "GMAC/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "u32", "data": "synthetic",
+        "vs_baseline": None, "dtype": {1: "u32", 2: "int8", 3: "fp4 (E2M1, exact for -1/0/+1) with fp32 accumulate"}[auto], "data": "synthetic",
         "config": {"workload": "TNN GEMM M=%d N=%d K=%d, uniform ternary, Packing 2, PReLU 0.5 fused" % (m, n, k),
                    "m": m, "n": n, "k": k},
-        "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
+        "roofline": roofline, "cpu_baseline": cpu,
+        "engine": lib.ENGINE_NAMES[auto], "engines": engines,
+        "roofline_valu_kernel": roofline_valu, "roofline_mfma_i8_kernel": mfma[lib.ENGINE_MFMA_I8],
+        "roofline_mfma_f4_kernel": mfma[lib.ENGINE_MFMA_F4], "extra": extra,
     }
     print(json.dumps(line), flush=True)
 

@@ -231,6 +231,47 @@ int64_t ftnn_mm_scratch_bytes(int engine, int type, int N, int OH, int OW, int K
     return mfma_fragment_bytes(f4, M, Kw) + mfma_fragment_bytes(f4, KN, Kw);
 }
 
+static int check_mfma_engine(int engine, int Kw) {
+    if (engine != FTNN_ENGINE_MFMA_I8 && engine != FTNN_ENGINE_MFMA_F4)
+        return fail(FTNN_EINVAL, "engine %d is not a matrix-core engine", engine);
+    if (engine == FTNN_ENGINE_MFMA_F4 && 64LL * Kw >= (1LL << 24))
+        return fail(FTNN_EINVAL, "K too long for exact fp32 accumulation; use the int8 engine");
+    return FTNN_OK;
+}
+
+int64_t ftnn_expand_bytes(int engine, int rows, int K) {
+    if (rows <= 0 || K <= 0 || (engine != FTNN_ENGINE_MFMA_I8 && engine != FTNN_ENGINE_MFMA_F4)) return 0;
+    return mfma_fragment_bytes(engine == FTNN_ENGINE_MFMA_F4, rows, round4(K));
+}
+
+int ftnn_expand_rows(int engine, int ternary, const int64_t* d_rows, int rows, int K, void* d_out,
+                     void* stream) {
+    if (rows <= 0 || K <= 0) return fail(FTNN_EINVAL, "non-positive dimension");
+    int rc = check_mfma_engine(engine, round4(K));
+    if (rc != FTNN_OK) return rc;
+    if (!d_rows || !d_out || !aligned16(d_rows) || !aligned16(d_out))
+        return fail(FTNN_EINVAL, "null or misaligned device pointer");
+    hipError_t e = launch_mfma_expand(engine == FTNN_ENGINE_MFMA_F4, ternary != 0, d_rows, rows, round4(K),
+                                      d_out, (hipStream_t)stream);
+    return e == hipSuccess ? FTNN_OK : hip_fail(e, "expand launch");
+}
+
+int ftnn_mm_expanded(int engine, int type, const void* d_a_exp, const void* d_b_exp, int N, int OH, int OW,
+                     int KN, int K, int K_unpack, float prelu_alpha, float* d_y, void* stream) {
+    if (type < kTNN || type > kBNN) return fail(FTNN_EINVAL, "unknown network type %d", type);
+    if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0)
+        return fail(FTNN_EINVAL, "non-positive GEMM dimension");
+    int rc = check_mfma_engine(engine, round4(K));
+    if (rc != FTNN_OK) return rc;
+    const int64_t M = (int64_t)N * OH * OW;
+    if (M > 0x7fffffffLL) return fail(FTNN_EINVAL, "more than 2^31-1 output rows");
+    if (!d_a_exp || !d_b_exp || !d_y || !aligned16(d_a_exp) || !aligned16(d_b_exp))
+        return fail(FTNN_EINVAL, "null or misaligned device pointer");
+    hipError_t e = launch_mfma_gemm(engine == FTNN_ENGINE_MFMA_F4, type, d_a_exp, d_b_exp, M, OH * OW, KN,
+                                    round4(K), K_unpack, prelu_alpha, d_y, (hipStream_t)stream);
+    return e == hipSuccess ? FTNN_OK : hip_fail(e, "mfma gemm launch");
+}
+
 int ftnn_mm_engine(int engine, int type, const int64_t* d_a, const int64_t* d_b, int N, int OH, int OW,
                    int KN, int K, int K_unpack, float prelu_alpha, float* d_y, void* d_scratch,
                    int64_t scratch_bytes, void* stream) {

@@ -29,6 +29,10 @@ hipError_t launch_mm(int type, const int64_t* d_a, const int64_t* d_b, int64_t M
 
 // ---- mfma_kernels.hip: matrix-core formulation (int8 or fp4 operands expanded into d_scratch) ----
 int64_t mfma_fragment_bytes(bool f4, int64_t rows, int Kw);
+hipError_t launch_mfma_expand(bool f4, bool ternary, const int64_t* d_rows, int rows, int Kw, void* d_out,
+                              hipStream_t st);
+hipError_t launch_mfma_gemm(bool f4, int type, const void* d_af, const void* d_bf, int64_t M, int OHW, int KN,
+                            int Kw, int K_unpack, float alpha, float* d_y, hipStream_t st);
 hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* d_b, int64_t M, int OHW,
                           int KN, int Kw, int K_unpack, float alpha, float* d_y, void* d_scratch,
                           hipStream_t st);

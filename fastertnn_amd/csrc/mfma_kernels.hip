@@ -240,42 +240,33 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
     for (; s + kNS < nstep; s++) step_body(s, std::true_type{});
     for (; s < nstep; s++) step_body(s, std::false_type{});
 
-    // accumulator e of block (a, b): P row = 32*prb + 8*(e/4) + 4*(lane/32) + e%4, Q row = 32*qrb + lane%32
+    // accumulator e of block (a, b): P row = 32*prb + 8*(e/4) + 4*(lane/32) + e%4, Q row = 32*qrb + lane%32.
+    // SWAP = false is only launched for OHW == 1 (row-major m x n result).
+    const bool le_form = form == 0;
 #pragma unroll
     for (int a = 0; a < 4; a++)
 #pragma unroll
         for (int b = 0; b < 4; b++) {
             const int q = (qrb0 + wx * 4 + b) * 32 + (lane & 31);
             const int pbase = (prb0 + wy * 4 + a) * 32 + 4 * (lane >> 5);
-            size_t qoff = 0;   // SWAP: q = i is fixed per block, hoist its image split
-            if (SWAP) {
+            size_t qoff;
+            if (SWAP) {   // q = i is fixed per block: split it into (image, pixel) once
                 const int img = q / OHW;
                 qoff = (size_t)img * KN * OHW + (q - img * OHW);
+            } else {
+                qoff = (size_t)q;
             }
+            const bool qok = q < (SWAP ? M : KN);
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 const int p = pbase + 8 * (e >> 2) + (e & 3);
-                const int i = SWAP ? q : p, j = SWAP ? p : q;
-                if (i < M && j < KN) {
-                    const int r = (int)acc[a][b][e] - bias;
-                    float f;
-                    if (form == 0) {
-                        f = (float)r;
-                        if (f <= 0) f *= alpha;
-                    } else {
-                        f = r >= 0 ? (float)r : alpha * r;
-                    }
-                    size_t o;
-                    if (SWAP) {
-                        o = qoff + (size_t)j * OHW;
-                    } else if (OHW == 1) {
-                        o = (size_t)i * KN + j;
-                    } else {
-                        const int img = i / OHW;
-                        o = ((size_t)img * KN + j) * OHW + (i - img * OHW);
-                    }
-                    Y[o] = f;
-                }
+                const int r = (int)acc[a][b][e] - bias;
+                const float fr = (float)r;
+                // form 0: scale when f <= 0 (a zero becomes 0 * alpha); form 1: scale when r < 0
+                const bool scale = le_form ? (fr <= 0.0f) : (r < 0);
+                const float f = scale ? fr * alpha : fr;
+                const size_t o = SWAP ? qoff + (size_t)p * OHW : (size_t)p * KN + qoff;
+                if (qok && p < (SWAP ? KN : M)) Y[o] = f;
             }
         }
 }
@@ -314,19 +305,19 @@ int64_t mfma_fragment_bytes(bool f4, int64_t rows, int Kw) {
     return ((rows + 31) / 32) * (int64_t)(f4 ? Kw : 2 * Kw) * 1024;
 }
 
-hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* d_b, int64_t M, int OHW,
-                          int KN, int Kw, int K_unpack, float alpha, float* d_y, void* d_scratch,
-                          hipStream_t st) {
-    const bool a_tern = (type == kTNN || type == kTBN), b_tern = (type == kTNN || type == kBTN);
-    const int G = Kw / 4, KB = f4 ? Kw : 2 * Kw;
-    uint4* Af = static_cast<uint4*>(d_scratch);
-    uint4* Bf = reinterpret_cast<uint4*>(static_cast<char*>(d_scratch) + mfma_fragment_bytes(f4, M, Kw));
-    const uint32_t* A = reinterpret_cast<const uint32_t*>(d_a);
-    const uint32_t* B = reinterpret_cast<const uint32_t*>(d_b);
-    hipError_t e = f4 ? launch_expand<true>(a_tern, A, (int)M, G, Af, st) : launch_expand<false>(a_tern, A, (int)M, G, Af, st);
-    if (e != hipSuccess) return e;
-    e = f4 ? launch_expand<true>(b_tern, B, KN, G, Bf, st) : launch_expand<false>(b_tern, B, KN, G, Bf, st);
-    if (e != hipSuccess) return e;
+hipError_t launch_mfma_expand(bool f4, bool ternary, const int64_t* d_rows, int rows, int Kw, void* d_out,
+                              hipStream_t st) {
+    const uint32_t* R = reinterpret_cast<const uint32_t*>(d_rows);
+    uint4* out = static_cast<uint4*>(d_out);
+    return f4 ? launch_expand<true>(ternary, R, rows, Kw / 4, out, st)
+              : launch_expand<false>(ternary, R, rows, Kw / 4, out, st);
+}
+
+hipError_t launch_mfma_gemm(bool f4, int type, const void* d_af, const void* d_bf, int64_t M, int OHW, int KN,
+                            int Kw, int K_unpack, float alpha, float* d_y, hipStream_t st) {
+    const int KB = f4 ? Kw : 2 * Kw;
+    const uint4* Af = static_cast<const uint4*>(d_af);
+    const uint4* Bf = static_cast<const uint4*>(d_bf);
     // BNN: the lanes past K_unpack are +1 in both operands and add 64*Kw - K_unpack to the dot
     // product; the reference's K_unpack - 2*popc(a^b) leaves them out (mm_p2_final_bnn_avx2.c:55-58)
     const int bias = type == kBNN ? 64 * Kw - K_unpack : 0;
@@ -338,6 +329,19 @@ hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* 
     }
     return swap ? launch_gemm<false, true>(Bf, Af, d_y, (int)M, KN, OHW, KB, bias, form, alpha, st)
                 : launch_gemm<false, false>(Af, Bf, d_y, (int)M, KN, OHW, KB, bias, form, alpha, st);
+}
+
+hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* d_b, int64_t M, int OHW,
+                          int KN, int Kw, int K_unpack, float alpha, float* d_y, void* d_scratch,
+                          hipStream_t st) {
+    const bool a_tern = (type == kTNN || type == kTBN), b_tern = (type == kTNN || type == kBTN);
+    void* Af = d_scratch;
+    void* Bf = static_cast<char*>(d_scratch) + mfma_fragment_bytes(f4, M, Kw);
+    hipError_t e = launch_mfma_expand(f4, a_tern, d_a, (int)M, Kw, Af, st);
+    if (e != hipSuccess) return e;
+    e = launch_mfma_expand(f4, b_tern, d_b, KN, Kw, Bf, st);
+    if (e != hipSuccess) return e;
+    return launch_mfma_gemm(f4, type, Af, Bf, M, OHW, KN, Kw, K_unpack, alpha, d_y, st);
 }
 
 }  // namespace ftnn

@@ -35,6 +35,10 @@ _L.ftnn_mm_scratch_bytes.restype = C.c_int64
 _L.ftnn_mm_scratch_bytes.argtypes = [C.c_int] * 7
 _L.ftnn_select_engine.argtypes = [C.c_int] * 6
 _L.ftnn_mm_engine.argtypes = [C.c_int, C.c_int, _vp, _vp] + [C.c_int] * 6 + [C.c_float, _vp, _vp, C.c_int64, _vp]
+_L.ftnn_expand_bytes.restype = C.c_int64
+_L.ftnn_expand_bytes.argtypes = [C.c_int] * 3
+_L.ftnn_expand_rows.argtypes = [C.c_int, C.c_int, _vp, C.c_int, C.c_int, _vp, _vp]
+_L.ftnn_mm_expanded.argtypes = [C.c_int, C.c_int, _vp, _vp] + [C.c_int] * 6 + [C.c_float, _vp, _vp]
 _L.ftnn_conv.argtypes = [C.c_int, _vp, _vp, _vp] + [C.c_int] * 11 + [C.c_float, _vp, _vp, _vp, _vp]
 _L.ftnn_pack_weights.argtypes = [C.c_int, _vp, _vp] + [C.c_int] * 4 + [_vp, _vp]
 _L.ftnn_pack_gemm_operand.argtypes = [_vp, C.c_int, C.c_int, _vp, _vp]
@@ -53,7 +57,7 @@ EXPORTS = ("tnns_conv", "tnns_gemm", "t2r_p2_opt", "b2r", "mm_tnn", "mm_tbn", "m
            "ftnn_last_error", "ftnn_version", "ftnn_out_dim", "ftnn_row_words",
            "ftnn_pack_scratch_bytes", "ftnn_quantize_im2row", "ftnn_mm", "ftnn_conv",
            "ftnn_pack_weights", "ftnn_pack_gemm_operand", "ftnn_select_engine", "ftnn_mm_scratch_bytes",
-           "ftnn_mm_engine")
+           "ftnn_mm_engine", "ftnn_expand_bytes", "ftnn_expand_rows", "ftnn_mm_expanded")
 
 ENGINE_AUTO, ENGINE_VALU, ENGINE_MFMA_I8, ENGINE_MFMA_F4 = 0, 1, 2, 3
 ENGINE_NAMES = {ENGINE_VALU: "valu", ENGINE_MFMA_I8: "mfma_i8", ENGINE_MFMA_F4: "mfma_f4"}
@@ -147,6 +151,25 @@ def mm_engine(engine, typ, a, b, n, oh, ow, kn, k, alpha, k_unpack=0, out=None, 
     sb = scratch.numel() * scratch.element_size() if scratch is not None else 0
     _check(_L.ftnn_mm_engine(engine, typ, _dev(a), _dev(b), n, oh, ow, kn, k, k_unpack, alpha,
                              _dev(out, torch.float32), sp, sb, _stream()))
+    return out
+
+
+def expand_rows(engine, rows_t, n_rows, k, ternary, out=None):
+    """ftnn_expand_rows: packed rows -> the operand format of a matrix-core engine."""
+    import torch
+    if out is None:
+        out = torch.empty(int(_L.ftnn_expand_bytes(engine, n_rows, k)), dtype=torch.uint8, device=rows_t.device)
+    _check(_L.ftnn_expand_rows(engine, int(ternary), _dev(rows_t), n_rows, k, _dev(out), _stream()))
+    return out
+
+
+def mm_expanded(engine, typ, a_exp, b_exp, n, oh, ow, kn, k, alpha, k_unpack=0, out=None):
+    """ftnn_mm_expanded: the matrix-core GEMM on two expanded operands."""
+    import torch
+    if out is None:
+        out = torch.empty((n, kn, oh, ow), dtype=torch.float32, device=a_exp.device)
+    _check(_L.ftnn_mm_expanded(engine, typ, _dev(a_exp), _dev(b_exp), n, oh, ow, kn, k, k_unpack, alpha,
+                               _dev(out, torch.float32), _stream()))
     return out
 
 

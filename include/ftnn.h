@@ -178,6 +178,20 @@ FTNN_API int ftnn_mm_engine(int engine, int type, const int64_t *d_a, const int6
                    void *d_scratch, int64_t scratch_bytes, void *stream);
 
 /*
+ * The two halves of a matrix-core GEMM, for callers that keep an operand expanded (weights
+ * are constant across calls).  ftnn_expand_rows turns `rows` packed rows of K words per
+ * plane (ternary != 0: Packing-2, else single-plane binary) into the operand format of
+ * `engine` (FTNN_ENGINE_MFMA_I8 or _F4), ftnn_expand_bytes() bytes at d_out;
+ * ftnn_mm_expanded multiplies two expanded operands and applies PReLU like ftnn_mm.
+ * No counterpart in the reference.
+ */
+FTNN_API int64_t ftnn_expand_bytes(int engine, int rows, int K);
+FTNN_API int ftnn_expand_rows(int engine, int ternary, const int64_t *d_rows, int rows, int K, void *d_out,
+                     void *stream);
+FTNN_API int ftnn_mm_expanded(int engine, int type, const void *d_a_exp, const void *d_b_exp, int N, int OH,
+                     int OW, int KN, int K, int K_unpack, float prelu_alpha, float *d_y, void *stream);
+
+/*
  * One conv layer on the device: ftnn_quantize_im2row then ftnn_mm
  * (src/tnns/tnns_cpu_mm_p2.c:6-80).  d_rows holds N*OH*OW packed rows.
  */
