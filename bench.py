@@ -107,12 +107,11 @@ def conv_latency(torch, lib, typ, shape, batch, seed, reps=20):
     wthr = torch.full((kn,), 0.5 if wt else 0.0, device="cuda")
     qw = lib.pack_weights(w, wthr, wt)
     oh, ow = lib.out_dim(ih, pad, kh, stride), lib.out_dim(iw, pad, kw, stride)
-    rows = torch.empty(batch * oh * ow * lib.row_words(c, kh, kw, at), dtype=torch.int64, device="cuda")
     scratch = torch.empty(lib.pack_scratch_bytes(batch, c, ih, iw, at), dtype=torch.uint8, device="cuda")
     y = torch.empty((batch, kn, oh, ow), device="cuda")
 
     def step():
-        lib.conv(typ, x, thr, qw, kn, kh, kw, pad, stride, 0.5, rows=rows, scratch=scratch, out=y)
+        lib.conv(typ, x, thr, qw, kn, kh, kw, pad, stride, 0.5, scratch=scratch, out=y)
 
     for _ in range(3):
         step()

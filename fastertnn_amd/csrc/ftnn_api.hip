@@ -307,17 +307,22 @@ int ftnn_mm_engine(int engine, int type, const int64_t* d_a, const int64_t* d_b,
 
 int ftnn_conv(int type, const float* d_x, const float* d_thr, const int64_t* d_qw, int N, int C,
               int H, int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride, int W_stride,
-              float prelu_alpha, int64_t* d_rows, void* d_scratch, float* d_y, void* stream) {
+              float prelu_alpha, void* d_scratch, float* d_y, void* stream) {
     if (type < kTNN || type > kBNN) return fail(FTNN_EINVAL, "unknown network type %d", type);
     int OH, OW;
     int rc = check_conv_shape(N, C, H, W, H_pad, W_pad, KH, KW, H_stride, W_stride, &OH, &OW);
     if (rc != FTNN_OK) return rc;
-    const int act_ternary = (type == kTNN || type == kTBN);
-    rc = ftnn_quantize_im2row(act_ternary, d_x, d_thr, N, C, H, W, H_pad, W_pad, KH, KW, H_stride,
-                              W_stride, d_rows, d_scratch, stream);
-    if (rc != FTNN_OK) return rc;
-    return ftnn_mm(type, d_rows, d_qw, N, OH, OW, KN, cpack_of(C) * KH * KW, C * KH * KW,
-                   prelu_alpha, d_y, stream);
+    if (KN <= 0) return fail(FTNN_EINVAL, "non-positive kernel count");
+    if (!d_x || !d_thr || !d_qw || !d_scratch || !d_y) return fail(FTNN_EINVAL, "null device pointer");
+    if (!aligned16(d_scratch) || !aligned16(d_qw))
+        return fail(FTNN_EINVAL, "d_scratch and d_qw must be 16-byte aligned");
+    if ((int64_t)N * OH * OW > 0x7fffffffLL) return fail(FTNN_EINVAL, "more than 2^31-1 output rows");
+    const bool act_ternary = (type == kTNN || type == kTBN);
+    hipError_t e = launch_quantize(act_ternary, d_x, d_thr, N, C, H, W, d_scratch, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "quantize launch");
+    const ConvGeom cg = {H, W, cpack_of(C), OH, OW, KW, cpack_of(C) * KH * KW, H_pad, W_pad, H_stride, W_stride};
+    e = launch_mm_implicit(type, d_scratch, d_qw, cg, N, KN, C * KH * KW, prelu_alpha, d_y, (hipStream_t)stream);
+    return e == hipSuccess ? FTNN_OK : hip_fail(e, "implicit-im2row mm launch");
 }
 
 int ftnn_pack_weights(int ternary, const float* d_w, const float* d_thr, int KN, int C, int KH,
@@ -385,13 +390,11 @@ void tnns_conv(testcase_t* t) {
     float* d_thr = (float*)upload(SLOT_THR, t->input_thresholds, (size_t)N * sizeof(float));
     int64_t* d_w = (int64_t*)upload(SLOT_W, t->quantized_kernel_packing2,
                                     (size_t)KN * ftnn_row_words(C, KH, KW, w_tern) * sizeof(int64_t));
-    int64_t* d_rows =
-        (int64_t*)dev_buf(SLOT_ROWS, rows * ftnn_row_words(C, KH, KW, act_tern) * sizeof(int64_t));
     void* d_scr = dev_buf(SLOT_SCRATCH, (size_t)ftnn_pack_scratch_bytes(N, C, H, W, act_tern));
     const size_t y_bytes = rows * KN * sizeof(float);
     float* d_y = (float*)dev_buf(SLOT_Y, y_bytes);
     if (ftnn_conv(type, d_x, d_thr, d_w, N, C, H, W, KN, KH, KW, t->paddingH, t->paddingW,
-                  t->strideH, t->strideW, t->preluAlpha, d_rows, d_scr, d_y,
+                  t->strideH, t->strideW, t->preluAlpha, d_scr, d_y,
                   host_stream()) != FTNN_OK)
         die("tnns_conv");
     float* y = (float*)host_alloc(y_bytes, false);

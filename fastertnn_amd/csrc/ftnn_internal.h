@@ -11,6 +11,12 @@ inline int cpack_of(int C) { return (C + 63) / 64; }
 inline int round4(int k) { return 4 * ((k + 3) / 4); }
 inline int out_dim(int in, int pad, int k, int stride) { return (in + 2 * pad - k) / stride + 1; }
 
+// geometry of one conv layer as the implicit-im2row GEMM needs it
+struct ConvGeom {
+    int H, W, CP, OH, OW, KW, K;   // K = C_pack*KH*KW words per plane before rounding
+    int H_pad, W_pad, H_stride, W_stride;
+};
+
 // record a failure text for ftnn_last_error(); returns `code`
 int fail(int code, const char* fmt, ...);
 
@@ -26,6 +32,13 @@ hipError_t launch_pack_gemm_operand(const float* d_x, int I, int J, int64_t* d_o
 hipError_t launch_mm(int type, const int64_t* d_a, const int64_t* d_b, int64_t M, int OHW, int KN,
                      int Kw /* words per plane, multiple of 4 */, int K_unpack, float alpha,
                      float* d_y, hipStream_t st);
+
+// GEMM straight from the channel-packed input P (no im2row matrix in memory)
+hipError_t launch_mm_implicit(int type, const void* d_p, const int64_t* d_b, const ConvGeom& cg, int N,
+                              int KN, int K_unpack, float alpha, float* d_y, hipStream_t st);
+// quantise only: fp32 NCHW -> P
+hipError_t launch_quantize(bool ternary, const float* d_x, const float* d_thr, int N, int C, int H, int W,
+                           void* d_p, hipStream_t st);
 
 // ---- mfma_kernels.hip: matrix-core formulation (int8 or fp4 operands expanded into d_scratch) ----
 int64_t mfma_fragment_bytes(bool f4, int64_t rows, int Kw);

@@ -94,11 +94,17 @@ __device__ __forceinline__ uint32_t popc4(const uint4& v) {
     return __popc(v.x) + __popc(v.y) + __popc(v.z) + __popc(v.w);
 }
 
-template <int MODE, int TM, int TN, int GC>
+// IMPL = true: implicit im2row.  A is then not a matrix of packed rows but the channel-packed
+// input P[n][pixel][ic] (one (sign, zero) pair of words, or one word for binary inputs, per
+// pixel and 64 channels); the staging step gathers word idx = (kh*KW + kw)*C_pack + ic of row
+// (n, oh, ow) from pixel (oh*s + kh - p, ow*s + kw - p) and applies the reference's fill rules
+// (src/tnns/ternarize2row_avx2.c:438-472, :748-755; src/tnns/binarize2row_avx2.c:151), so the
+// im2row matrix is never written to memory.
+template <int MODE, int TM, int TN, int GC, bool IMPL>
 __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
                                             const uint32_t* __restrict__ B,
                                             float* __restrict__ Y, int M, int KN, int OHW, int G,
-                                            int K_unpack, float alpha) {
+                                            int K_unpack, float alpha, ConvGeom cg) {
     using T = Traits<MODE>;
     constexpr int BM = 64 * TM;
     constexpr int AG = T::kAGroup, BG = T::kBGroup;
@@ -137,41 +143,84 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
 #pragma unroll
     for (int b = 0; b < TN; b++) bcol[b] = B + (size_t)min(col0 + b, KN - 1) * RDB;
 
-    // staging map: pass `it` of this thread moves quad sq of tile row sr + it*RPI
-    const int sq = tid % QPR, sr = tid / QPR;
-    const bool stager = (QUADS % 256 == 0) || (tid < QUADS);
+    // staging map (explicit rows): pass `it` of this thread moves quad sq of tile row sr + it*RPI
+    const int sq = IMPL ? (tid & 3) : tid % QPR, sr = IMPL ? (tid >> 2) : tid / QPR;
+    const bool stager = IMPL || (QUADS % 256 == 0) || (tid < QUADS);
     const uint32_t* ap[IT];
-#pragma unroll
-    for (int it = 0; it < IT; it++)
-        ap[it] = A + (size_t)min(row0 + sr + it * RPI, (int64_t)M - 1) * RDA + sq * 4;
-    uint32_t* const lw = &lds[0][0] + sr * LDW + sq * 4;
+    uint32_t* const lw = &lds[0][0] + sr * LDW + sq * (IMPL ? 2 : 4);
     uint4 stage[IT];
-
-    const int nchunk = (G + GC - 1) / GC;
-    {
-        const bool on = stager && sq < min(GC, G) * (AG / 4);
+    // staging map (implicit im2row): thread = (word sq of the group, tile row sr + it*64)
+    constexpr int ITI = IMPL ? TM : 1;
+    int ih0[ITI], iw0[ITI];
+    size_t pix0[ITI];
+    ulonglong2 istage[ITI];
+    static_assert(!IMPL || GC == 1, "implicit im2row stages one group per chunk");
+    if (IMPL) {
+#pragma unroll
+        for (int it = 0; it < ITI; it++) {
+            const int64_t r = min(row0 + sr + it * 64, (int64_t)M - 1);
+            const int64_t n = r / OHW;
+            const int pix = (int)(r - n * OHW);
+            const int oh = pix / cg.OW, ow = pix - oh * cg.OW;
+            ih0[it] = oh * cg.H_stride - cg.H_pad;
+            iw0[it] = ow * cg.W_stride - cg.W_pad;
+            pix0[it] = (size_t)n * cg.H * cg.W;
+        }
+    } else {
 #pragma unroll
         for (int it = 0; it < IT; it++)
-            stage[it] = on ? *reinterpret_cast<const uint4*>(ap[it]) : make_uint4(0, 0, 0, 0);
-        if (stager) {
+            ap[it] = A + (size_t)min(row0 + sr + it * RPI, (int64_t)M - 1) * RDA + sq * 4;
+    }
+    // issue the global loads of group-chunk starting at group g0 into the staging registers
+    auto fetch = [&](int g0) {
+        if (IMPL) {
+            const int idx = g0 * 4 + sq;
+            const bool valid = idx < cg.K;
+            const int tap = idx / cg.CP, ic = idx - tap * cg.CP;
+            const int kh = tap / cg.KW, kw = tap - kh * cg.KW;
+#pragma unroll
+            for (int it = 0; it < ITI; it++) {
+                const int ih = ih0[it] + kh, iw = iw0[it] + kw;
+                const bool in = valid && ih >= 0 && ih < cg.H && iw >= 0 && iw < cg.W;
+                const size_t o = (pix0[it] + (size_t)(in ? ih * cg.W + iw : 0)) * cg.CP + (in ? ic : 0);
+                if (T::kATern) {
+                    istage[it] = in ? reinterpret_cast<const ulonglong2*>(A)[o] : make_ulonglong2(0ull, ~0ull);
+                } else {
+                    istage[it].x = in ? reinterpret_cast<const unsigned long long*>(A)[o] : 0ull;
+                }
+            }
+        } else {
+            const bool on = stager && sq < min(GC, G - g0) * (AG / 4);
 #pragma unroll
             for (int it = 0; it < IT; it++)
-                *reinterpret_cast<uint4*>(lw + it * RPI * LDW) = stage[it];
+                stage[it] = on ? *reinterpret_cast<const uint4*>(ap[it] + (size_t)g0 * AG) : make_uint4(0, 0, 0, 0);
         }
-    }
+    };
+    // write the staging registers into LDS buffer `buf`
+    auto commit = [&](int buf) {
+        uint32_t* l = lw + buf * (BM * LDW);
+        if (IMPL) {
+#pragma unroll
+            for (int it = 0; it < ITI; it++) {
+                *reinterpret_cast<unsigned long long*>(l + it * 64 * LDW) = istage[it].x;
+                if (T::kATern) *reinterpret_cast<unsigned long long*>(l + it * 64 * LDW + 8) = istage[it].y;
+            }
+        } else if (stager) {
+#pragma unroll
+            for (int it = 0; it < IT; it++) *reinterpret_cast<uint4*>(l + it * RPI * LDW) = stage[it];
+        }
+    };
+
+    const int nchunk = (G + GC - 1) / GC;
+    fetch(0);
+    commit(0);
     __syncthreads();
 
     for (int c = 0; c < nchunk; c++) {
         const int g0 = c * GC;
         const int gc = min(GC, G - g0);
         const bool more = c + 1 < nchunk;
-        if (more) {  // issue the global loads of the next chunk; they land after the arithmetic
-            const bool on = stager && sq < min(GC, G - g0 - GC) * (AG / 4);
-#pragma unroll
-            for (int it = 0; it < IT; it++)
-                stage[it] = on ? *reinterpret_cast<const uint4*>(ap[it] + (size_t)(g0 + GC) * AG)
-                               : make_uint4(0, 0, 0, 0);
-        }
+        if (more) fetch(g0 + GC);  // the loads of the next chunk land after the arithmetic
         const uint32_t* lr = &lds[c & 1][0];
         for (int g = 0; g < gc; g++) {
             uint4 sa0[TM], sa1[TM], za0[TM], za1[TM];
@@ -216,12 +265,7 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
                 cur = nxt;
             }
         }
-        if (more && stager) {
-            uint32_t* lwn = lw + ((c + 1) & 1) * (BM * LDW);
-#pragma unroll
-            for (int it = 0; it < IT; it++)
-                *reinterpret_cast<uint4*>(lwn + it * RPI * LDW) = stage[it];
-        }
+        if (more) commit((c + 1) & 1);
         __syncthreads();
     }
 
@@ -257,29 +301,29 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
     }
 }
 
-template <int MODE, int TM, int TN, int GC>
+template <int MODE, int TM, int TN, int GC, bool IMPL>
 hipError_t launch_cfg(const uint32_t* A, const uint32_t* B, float* Y, int64_t M, int KN, int OHW,
-                      int G, int K_unpack, float alpha, hipStream_t st) {
+                      int G, int K_unpack, float alpha, const ConvGeom& cg, hipStream_t st) {
     const int64_t gx = (M + 64 * TM - 1) / (64 * TM);
     const int64_t gy = (KN + 4 * TN - 1) / (4 * TN);
     if (gx > 0x7fffffffLL || gy > 65535) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((k_mm<MODE, TM, TN, GC>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
-                       A, B, Y, (int)M, KN, OHW, G, K_unpack, alpha);
+    hipLaunchKernelGGL((k_mm<MODE, TM, TN, GC, IMPL>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
+                       A, B, Y, (int)M, KN, OHW, G, K_unpack, alpha, cg);
     return hipGetLastError();
 }
 
-template <int MODE>
+template <int MODE, bool IMPL>
 hipError_t launch_mode(const uint32_t* A, const uint32_t* B, float* Y, int64_t M, int KN, int OHW,
-                       int G, int K_unpack, float alpha, hipStream_t st) {
+                       int G, int K_unpack, float alpha, const ConvGeom& cg, hipStream_t st) {
     // Tile choice (measured on MI355X): 128 x 32 tiles once they give each of the 256 CUs
     // a dozen workgroups; layer-sized problems are one or two waves of workgroups, where
     // smaller tiles finish sooner.
     auto wgs = [&](int tm, int tn) {
         return ((M + 64 * tm - 1) / (64 * tm)) * ((KN + 4 * tn - 1) / (4 * tn));
     };
-    if (wgs(2, 8) >= 3072) return launch_cfg<MODE, 2, 8, 1>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, st);
-    if (wgs(1, 4) >= 2048) return launch_cfg<MODE, 1, 4, 1>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, st);
-    return launch_cfg<MODE, 1, 2, 1>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, st);
+    if (wgs(2, 8) >= 3072) return launch_cfg<MODE, 2, 8, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+    if (wgs(1, 4) >= 2048) return launch_cfg<MODE, 1, 4, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+    return launch_cfg<MODE, 1, 2, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
 }
 
 }  // namespace
@@ -289,11 +333,28 @@ hipError_t launch_mm(int type, const int64_t* d_a, const int64_t* d_b, int64_t M
     const uint32_t* A = reinterpret_cast<const uint32_t*>(d_a);
     const uint32_t* B = reinterpret_cast<const uint32_t*>(d_b);
     const int G = Kw / 4;
+    const ConvGeom cg = {};
     switch (type) {
-        case kTNN: return launch_mode<kTNN>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, st);
-        case kTBN: return launch_mode<kTBN>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, st);
-        case kBTN: return launch_mode<kBTN>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, st);
-        case kBNN: return launch_mode<kBNN>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, st);
+        case kTNN: return launch_mode<kTNN, false>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+        case kTBN: return launch_mode<kTBN, false>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+        case kBTN: return launch_mode<kBTN, false>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+        case kBNN: return launch_mode<kBNN, false>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+    }
+    return hipErrorInvalidValue;
+}
+
+hipError_t launch_mm_implicit(int type, const void* d_p, const int64_t* d_b, const ConvGeom& cg, int N,
+                              int KN, int K_unpack, float alpha, float* d_y, hipStream_t st) {
+    const uint32_t* A = static_cast<const uint32_t*>(d_p);
+    const uint32_t* B = reinterpret_cast<const uint32_t*>(d_b);
+    const int OHW = cg.OH * cg.OW;
+    const int64_t M = (int64_t)N * OHW;
+    const int G = round4(cg.K) / 4;
+    switch (type) {
+        case kTNN: return launch_mode<kTNN, true>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+        case kTBN: return launch_mode<kTBN, true>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+        case kBTN: return launch_mode<kBTN, true>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+        case kBNN: return launch_mode<kBNN, true>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
     }
     return hipErrorInvalidValue;
 }

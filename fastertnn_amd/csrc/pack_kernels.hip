@@ -29,46 +29,50 @@ __device__ __forceinline__ int64_t p2_pos(int64_t idx, int plane) {
 }
 
 // ---------------------------------------------------------------- quantise
-// lanes along pixels: grid (ceil(HW/256), C_pack, N)
+// Block = 32 consecutive pixels x 8 channel octets of one 64-channel word.  The 32 lanes
+// of an octet read 128 contiguous bytes of one channel plane (coalesced); every thread
+// thresholds 8 channels into one byte per plane, the bytes meet in LDS and 32 threads
+// write the finished words.  grid (ceil(HW/32), C_pack, N).
 template <bool TERN>
 __global__ __launch_bounds__(256) void k_quantize_pixels(const float* __restrict__ x,
                                                          const float* __restrict__ thr, int C,
                                                          int HW, int CP,
                                                          unsigned long long* __restrict__ P) {
-    const int p = blockIdx.x * 256 + threadIdx.x;
+    __shared__ unsigned long long s_neg[32], s_nz[32];
+    const int px = threadIdx.x & 31, oct = threadIdx.x >> 5;
+    const int p = blockIdx.x * 32 + px;
     const int ic = blockIdx.y, n = blockIdx.z;
-    if (p >= HW) return;
     const float t = thr[n];
-    const int nb = min(64, C - ic * 64);
-    const float* xp = x + ((size_t)n * C + (size_t)ic * 64) * HW + p;
-    uint32_t neg[2] = {0u, 0u}, nz[2] = {0u, 0u};
+    const int c0 = ic * 64 + oct * 8;
+    uint32_t neg = 0u, nz = 0u;
+    if (p < HW) {
+        const float* xp = x + ((size_t)n * C + c0) * HW + p;
+        float v[8];
 #pragma unroll
-    for (int half = 0; half < 2; half++) {
-#pragma unroll 8
-        for (int bit = 0; bit < 32; bit++) {
-            const int c = half * 32 + bit;
-            if (c < nb) {
-                const float v = xp[(size_t)c * HW];
+        for (int j = 0; j < 8; j++) v[j] = (c0 + j < C) ? xp[(size_t)j * HW] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            if (c0 + j < C) {
                 if (TERN) {
                     // strict compares, src/tnns/ternarize2row_avx2.c:443-449
-                    const bool isneg = v < -t;
-                    const bool ispos = v > t;
-                    neg[half] |= (isneg ? 1u : 0u) << bit;
-                    nz[half] |= ((isneg || ispos) ? 1u : 0u) << bit;
+                    const bool isneg = v[j] < -t;
+                    const bool ispos = v[j] > t;
+                    neg |= (isneg ? 1u : 0u) << j;
+                    nz |= ((isneg || ispos) ? 1u : 0u) << j;
                 } else {
                     // src/tnns/binarize2row_avx2.c:19-21
-                    neg[half] |= (v < t ? 1u : 0u) << bit;
+                    neg |= (v[j] < t ? 1u : 0u) << j;
                 }
             }
         }
     }
-    const size_t o = ((size_t)n * HW + p) * CP + ic;
-    const unsigned long long s = ((unsigned long long)neg[1] << 32) | neg[0];
-    if (TERN) {
-        const unsigned long long z = ~(((unsigned long long)nz[1] << 32) | nz[0]);
-        reinterpret_cast<ulonglong2*>(P)[o] = make_ulonglong2(s, z);
-    } else {
-        P[o] = s;
+    reinterpret_cast<unsigned char*>(s_neg)[px * 8 + oct] = (unsigned char)neg;
+    if (TERN) reinterpret_cast<unsigned char*>(s_nz)[px * 8 + oct] = (unsigned char)nz;
+    __syncthreads();
+    if (threadIdx.x < 32 && p < HW) {
+        const size_t o = ((size_t)n * HW + p) * CP + ic;
+        if (TERN) reinterpret_cast<ulonglong2*>(P)[o] = make_ulonglong2(s_neg[px], ~s_nz[px]);
+        else P[o] = s_neg[px];
     }
 }
 
@@ -203,13 +207,10 @@ __global__ __launch_bounds__(256) void k_pack_weights(const float* __restrict__ 
 
 }  // namespace
 
-hipError_t launch_quantize_im2row(bool ternary, const float* d_x, const float* d_thr, int N, int C,
-                                  int H, int W, int H_pad, int W_pad, int kH, int kW, int H_stride,
-                                  int W_stride, int64_t* d_out, void* d_scratch, hipStream_t st) {
+hipError_t launch_quantize(bool ternary, const float* d_x, const float* d_thr, int N, int C, int H, int W,
+                           void* d_p, hipStream_t st) {
     const int CP = cpack_of(C), HW = H * W;
-    const int OH = out_dim(H, H_pad, kH, H_stride), OW = out_dim(W, W_pad, kW, W_stride);
-    const int K = CP * kH * kW, Kw = round4(K);
-    unsigned long long* P = static_cast<unsigned long long*>(d_scratch);
+    unsigned long long* P = static_cast<unsigned long long*>(d_p);
     if (HW == 1) {
         // 64 consecutive floats are one word: wavefront ballot
         dim3 grid(N, (CP + 3) / 4);
@@ -220,7 +221,7 @@ hipError_t launch_quantize_im2row(bool ternary, const float* d_x, const float* d
             hipLaunchKernelGGL((k_quantize_ballot<1, false>), grid, dim3(256), 0, st, d_x, d_thr, C,
                                CP, P);
     } else {
-        dim3 grid((HW + 255) / 256, CP, N);
+        dim3 grid((HW + 31) / 32, CP, N);
         if (ternary)
             hipLaunchKernelGGL((k_quantize_pixels<true>), grid, dim3(256), 0, st, d_x, d_thr, C, HW,
                                CP, P);
@@ -228,7 +229,17 @@ hipError_t launch_quantize_im2row(bool ternary, const float* d_x, const float* d
             hipLaunchKernelGGL((k_quantize_pixels<false>), grid, dim3(256), 0, st, d_x, d_thr, C,
                                HW, CP, P);
     }
-    hipError_t e = hipGetLastError();
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_im2row(bool ternary, const float* d_x, const float* d_thr, int N, int C,
+                                  int H, int W, int H_pad, int W_pad, int kH, int kW, int H_stride,
+                                  int W_stride, int64_t* d_out, void* d_scratch, hipStream_t st) {
+    const int CP = cpack_of(C);
+    const int OH = out_dim(H, H_pad, kH, H_stride), OW = out_dim(W, W_pad, kW, W_stride);
+    const int K = CP * kH * kW, Kw = round4(K);
+    unsigned long long* P = static_cast<unsigned long long*>(d_scratch);
+    hipError_t e = launch_quantize(ternary, d_x, d_thr, N, C, H, W, d_scratch, st);
     if (e != hipSuccess) return e;
     const int64_t total = (int64_t)N * OH * OW * Kw;
     const unsigned blocks = (unsigned)((total + 255) / 256);

@@ -39,7 +39,7 @@ _L.ftnn_expand_bytes.restype = C.c_int64
 _L.ftnn_expand_bytes.argtypes = [C.c_int] * 3
 _L.ftnn_expand_rows.argtypes = [C.c_int, C.c_int, _vp, C.c_int, C.c_int, _vp, _vp]
 _L.ftnn_mm_expanded.argtypes = [C.c_int, C.c_int, _vp, _vp] + [C.c_int] * 6 + [C.c_float, _vp, _vp]
-_L.ftnn_conv.argtypes = [C.c_int, _vp, _vp, _vp] + [C.c_int] * 11 + [C.c_float, _vp, _vp, _vp, _vp]
+_L.ftnn_conv.argtypes = [C.c_int, _vp, _vp, _vp] + [C.c_int] * 11 + [C.c_float, _vp, _vp, _vp]
 _L.ftnn_pack_weights.argtypes = [C.c_int, _vp, _vp] + [C.c_int] * 4 + [_vp, _vp]
 _L.ftnn_pack_gemm_operand.argtypes = [_vp, C.c_int, C.c_int, _vp, _vp]
 for _n in ("t2r_p2_opt", "b2r"):
@@ -173,7 +173,7 @@ def mm_expanded(engine, typ, a_exp, b_exp, n, oh, ow, kn, k, alpha, k_unpack=0, 
     return out
 
 
-def conv(typ, x, thr, qw, kn, kh, kw, pad, stride, alpha, rows=None, scratch=None, out=None):
+def conv(typ, x, thr, qw, kn, kh, kw, pad, stride, alpha, scratch=None, out=None):
     """One conv layer (tnn_conv_p2 & co.) on device tensors."""
     import torch
     n, c, h, w = x.shape
@@ -181,15 +181,12 @@ def conv(typ, x, thr, qw, kn, kh, kw, pad, stride, alpha, rows=None, scratch=Non
     if oh <= 0 or ow <= 0:
         raise FtnnError("kernel larger than padded input")
     tern = act_is_ternary(typ)
-    if rows is None:
-        rows = torch.empty(n * oh * ow * row_words(c, kh, kw, tern), dtype=torch.int64, device=x.device)
     if scratch is None:
         scratch = torch.empty(pack_scratch_bytes(n, c, h, w, tern), dtype=torch.uint8, device=x.device)
     if out is None:
         out = torch.empty((n, kn, oh, ow), dtype=torch.float32, device=x.device)
     _check(_L.ftnn_conv(typ, _dev(x, torch.float32), _dev(thr, torch.float32), _dev(qw), n, c, h, w, kn, kh,
-                        kw, pad, pad, stride, stride, alpha, _dev(rows), _dev(scratch),
-                        _dev(out, torch.float32), _stream()))
+                        kw, pad, pad, stride, stride, alpha, _dev(scratch), _dev(out, torch.float32), _stream()))
     return out
 
 

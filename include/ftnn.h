@@ -192,13 +192,14 @@ FTNN_API int ftnn_mm_expanded(int engine, int type, const void *d_a_exp, const v
                      int OW, int KN, int K, int K_unpack, float prelu_alpha, float *d_y, void *stream);
 
 /*
- * One conv layer on the device: ftnn_quantize_im2row then ftnn_mm
- * (src/tnns/tnns_cpu_mm_p2.c:6-80).  d_rows holds N*OH*OW packed rows.
+ * One conv layer on the device (src/tnns/tnns_cpu_mm_p2.c:6-80): the input is quantised
+ * once into d_scratch (ftnn_pack_scratch_bytes() bytes) and the GEMM gathers its im2row
+ * operand from there, so the im2row matrix of t2r_p2_opt / b2r is never written to memory.
+ * Same result as ftnn_quantize_im2row followed by ftnn_mm.
  */
 FTNN_API int ftnn_conv(int type, const float *d_x, const float *d_thr, const int64_t *d_qw, int N, int C,
               int H, int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride,
-              int W_stride, float prelu_alpha, int64_t *d_rows, void *d_scratch, float *d_y,
-              void *stream);
+              int W_stride, float prelu_alpha, void *d_scratch, float *d_y, void *stream);
 
 /*
  * Weight packers on the device: fp32 (KN,C,KH,KW) -> Packing-2 rows.  ternary != 0 is

@@ -78,7 +78,7 @@ def test_bad_arguments_are_rejected_without_touching_the_device():
     # kernel larger than the padded input
     assert L.ftnn_quantize_im2row(1, p, p, 1, 8, 2, 2, 0, 0, 3, 3, 1, 1, p, p, None) == -1
     assert L.ftnn_quantize_im2row(1, p, p, 1, 8, 4, 4, 0, 0, 3, 3, 0, 1, p, p, None) == -1  # stride 0
-    assert L.ftnn_conv(9, p, p, p, 1, 8, 4, 4, 4, 3, 3, 1, 1, 1, 1, 0.5, p, p, p, None) == -1
+    assert L.ftnn_conv(9, p, p, p, 1, 8, 4, 4, 4, 3, 3, 1, 1, 1, 1, 0.5, p, p, None) == -1
     assert L.ftnn_pack_weights(1, p, p, 0, 8, 3, 3, p, None) == -1
 
 
