@@ -24,6 +24,8 @@
 //     distinct banks.
 // A workgroup is 4 wavefronts sharing one A tile of 64*TM rows; wavefront w
 // computes columns [w*TN, (w+1)*TN) of the workgroup's 4*TN columns.
+#include <stdlib.h>
+
 #include "ftnn_internal.h"
 
 namespace ftnn {
@@ -158,10 +160,10 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
     if (IMPL) {
 #pragma unroll
         for (int it = 0; it < ITI; it++) {
-            const int64_t r = min(row0 + sr + it * 64, (int64_t)M - 1);
-            const int64_t n = r / OHW;
-            const int pix = (int)(r - n * OHW);
-            const int oh = pix / cg.OW, ow = pix - oh * cg.OW;
+            const uint32_t r = (uint32_t)min(row0 + sr + it * 64, (int64_t)M - 1);
+            const uint32_t n = r / (uint32_t)OHW;
+            const uint32_t pix = r - n * (uint32_t)OHW;
+            const int oh = (int)(pix / (uint32_t)cg.OW), ow = (int)pix - oh * cg.OW;
             ih0[it] = oh * cg.H_stride - cg.H_pad;
             iw0[it] = ow * cg.W_stride - cg.W_pad;
             pix0[it] = (size_t)n * cg.H * cg.W;
@@ -171,13 +173,31 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
         for (int it = 0; it < IT; it++)
             ap[it] = A + (size_t)min(row0 + sr + it * RPI, (int64_t)M - 1) * RDA + sq * 4;
     }
+    // word idx = 4*g + sq of the group being fetched, kept as (kh, kw, ic) and advanced by 4 words per
+    // chunk without divisions (chunks are fetched in order, one group each)
+    int f_ic = 0, f_kh = 0, f_kw = 0;
+    if (IMPL) {
+        const int tap = sq / cg.CP;
+        f_ic = sq - tap * cg.CP;
+        f_kh = tap / cg.KW;
+        f_kw = tap - f_kh * cg.KW;
+    }
     // issue the global loads of group-chunk starting at group g0 into the staging registers
     auto fetch = [&](int g0) {
         if (IMPL) {
-            const int idx = g0 * 4 + sq;
-            const bool valid = idx < cg.K;
-            const int tap = idx / cg.CP, ic = idx - tap * cg.CP;
-            const int kh = tap / cg.KW, kw = tap - kh * cg.KW;
+            const bool valid = g0 * 4 + sq < cg.K;
+            const int ic = f_ic, kh = f_kh, kw = f_kw;
+            f_ic += 4;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {   // at most 4 wraps (C_pack = 1); one when C_pack >= 4
+                if (f_ic >= cg.CP) {
+                    f_ic -= cg.CP;
+                    if (++f_kw == cg.KW) {
+                        f_kw = 0;
+                        f_kh++;
+                    }
+                }
+            }
 #pragma unroll
             for (int it = 0; it < ITI; it++) {
                 const int ih = ih0[it] + kh, iw = iw0[it] + kw;
@@ -274,8 +294,8 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
     for (int a = 0; a < TM; a++) {
         const int64_t i = row0 + lane + 64 * a;
         if (i < M) {
-            const int64_t img = i / OHW;
-            const int pix = (int)(i - img * OHW);
+            const uint32_t img = (uint32_t)i / (uint32_t)OHW;
+            const uint32_t pix = (uint32_t)i - img * (uint32_t)OHW;
 #pragma unroll
             for (int b = 0; b < TN; b++) {
                 const int j = col0 + b;
@@ -321,6 +341,10 @@ hipError_t launch_mode(const uint32_t* A, const uint32_t* B, float* Y, int64_t M
     auto wgs = [&](int tm, int tn) {
         return ((M + 64 * tm - 1) / (64 * tm)) * ((KN + 4 * tn - 1) / (4 * tn));
     };
+    static const char* force = getenv("FTNN_MM_TILE");   // tuning aid: "28", "14" or "12" forces a tile
+    if (force && force[0] == '2') return launch_cfg<MODE, 2, 8, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+    if (force && force[1] == '4') return launch_cfg<MODE, 1, 4, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+    if (force && force[1] == '2') return launch_cfg<MODE, 1, 2, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
     if (wgs(2, 8) >= 3072) return launch_cfg<MODE, 2, 8, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
     if (wgs(1, 4) >= 2048) return launch_cfg<MODE, 1, 4, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
     return launch_cfg<MODE, 1, 2, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
