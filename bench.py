@@ -137,6 +137,57 @@ def conv_latency(torch, lib, typ, shape, batch, seed, reps=20):
     return out
 
 
+RESNET18_LIKE = [  # (C, IH, IW, KN, KW, KH, pad, stride): stem, four stages with stride-2 transitions, FC as 1x1
+    (3, 224, 224, 64, 7, 7, 3, 2), (64, 112, 112, 64, 3, 3, 1, 2),
+    (64, 56, 56, 64, 3, 3, 1, 1), (64, 56, 56, 64, 3, 3, 1, 1), (64, 56, 56, 64, 3, 3, 1, 1), (64, 56, 56, 64, 3, 3, 1, 1),
+    (64, 56, 56, 128, 3, 3, 1, 2), (128, 28, 28, 128, 3, 3, 1, 1), (128, 28, 28, 128, 3, 3, 1, 1), (128, 28, 28, 128, 3, 3, 1, 1),
+    (128, 28, 28, 256, 3, 3, 1, 2), (256, 14, 14, 256, 3, 3, 1, 1), (256, 14, 14, 256, 3, 3, 1, 1), (256, 14, 14, 256, 3, 3, 1, 1),
+    (256, 14, 14, 512, 3, 3, 1, 2), (512, 7, 7, 512, 3, 3, 1, 1), (512, 7, 7, 512, 3, 3, 1, 1), (512, 7, 7, 512, 3, 3, 1, 1),
+    (512, 7, 7, 1000, 1, 1, 0, 1),
+]
+
+
+def e2e_latency(torch, lib, batch, reps=10):
+    """the batch-32 ResNet-18-like TNN stack chained on the device (eager launches and HIP-graph
+    replay), and the same chain through the reference's tnns_conv on one host core"""
+    import numpy as np
+    from fastertnn_amd import TNN
+    g = torch.Generator(device="cuda")
+    g.manual_seed(6)
+    x = torch.randn((batch, 3, 224, 224), generator=g, device="cuda")
+    layers = []
+    for (c, ih, iw, kn, kw, kh, pad, stride) in RESNET18_LIKE:
+        w = torch.randint(-1, 2, (kn, c, kh, kw), generator=g, device="cuda", dtype=torch.int8).float()
+        qw = lib.pack_weights(w, torch.full((kn,), 0.5, device="cuda"), True)
+        layers.append(dict(type=TNN, shape=(c, ih, iw, kn, kw, kh, pad, stride), threshold=0.5, alpha=0.5, qw=qw))
+    net = lib.Net(batch, layers)
+    y = torch.empty(net.out_shape, device="cuda")
+    macs = sum(batch * lib.out_dim(ih, p, kh, s) * lib.out_dim(iw, p, kw, s) * kn * c * kh * kw
+               for (c, ih, iw, kn, kw, kh, p, s) in RESNET18_LIKE)
+    out = {"layers": len(layers), "batch": batch, "gmac": round(macs / 1e9, 2)}
+    st = torch.cuda.Stream()
+    with torch.cuda.stream(st):
+        for graph, key in ((False, "eager_ms"), (True, "graph_ms")):
+            for _ in range(3):
+                net.run(x, out=y, graph=graph)
+            t = sorted(event_times(torch, lambda: net.run(x, out=y, graph=graph), reps))[reps // 2]
+            out[key] = round(t, 4)
+    st.synchronize()
+    from oracle import ftnn_oracle as O
+    if O.Reference.available():
+        ref = O.Reference()
+        xh = x.cpu().numpy()
+        thr = np.full(batch, 0.5, np.float32)
+        t0 = time.perf_counter()
+        for l in layers:
+            c, ih, iw, kn, kw, kh, pad, stride = l["shape"]
+            xh = ref.conv(TNN, xh, thr, O.aligned_copy(l["qw"].cpu().numpy()), kn, kh, kw, pad, stride, 0.5)
+        out["cpu_ms"] = round((time.perf_counter() - t0) * 1e3, 1)
+        out["bit_exact_vs_reference"] = bool(y.cpu().numpy().tobytes() == np.ascontiguousarray(xh).tobytes())
+    net.close()
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -250,6 +301,7 @@ def main():
             "tnn_conv_b1_c256_56x56_k3": conv_latency(torch, lib, TNN, (256, 56, 56, 256, 3, 3, 1, 1), 1, 2),
             "tbn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, TBN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 3),
             "btn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, BTN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 4),
+            "tnn_resnet18_like_b32_e2e": e2e_latency(torch, lib, 32),
         }
 
     line = {

@@ -57,7 +57,8 @@ EXPORTS = ("tnns_conv", "tnns_gemm", "t2r_p2_opt", "b2r", "mm_tnn", "mm_tbn", "m
            "ftnn_last_error", "ftnn_version", "ftnn_out_dim", "ftnn_row_words",
            "ftnn_pack_scratch_bytes", "ftnn_quantize_im2row", "ftnn_mm", "ftnn_conv",
            "ftnn_pack_weights", "ftnn_pack_gemm_operand", "ftnn_select_engine", "ftnn_mm_scratch_bytes",
-           "ftnn_mm_engine", "ftnn_expand_bytes", "ftnn_expand_rows", "ftnn_mm_expanded")
+           "ftnn_mm_engine", "ftnn_expand_bytes", "ftnn_expand_rows", "ftnn_mm_expanded",
+           "ftnn_net_create", "ftnn_net_destroy", "ftnn_net_output_elems", "ftnn_net_run")
 
 ENGINE_AUTO, ENGINE_VALU, ENGINE_MFMA_I8, ENGINE_MFMA_F4 = 0, 1, 2, 3
 ENGINE_NAMES = {ENGINE_VALU: "valu", ENGINE_MFMA_I8: "mfma_i8", ENGINE_MFMA_F4: "mfma_f4"}
@@ -207,6 +208,58 @@ def pack_gemm_operand(x):
     out = torch.empty(max(i * j // 32, 1), dtype=torch.int64, device=x.device)
     _check(_L.ftnn_pack_gemm_operand(_dev(x, torch.float32), i, j, _dev(out), _stream()))
     return out
+
+
+class LayerDesc(C.Structure):
+    """ftnn_layer_t"""
+    _fields_ = [("type", C.c_int), ("C", C.c_int), ("H", C.c_int), ("W", C.c_int), ("KN", C.c_int),
+                ("KH", C.c_int), ("KW", C.c_int), ("pad", C.c_int), ("stride", C.c_int),
+                ("threshold", C.c_float), ("prelu_alpha", C.c_float), ("d_qw", _vp)]
+
+
+_L.ftnn_net_create.restype = _vp
+_L.ftnn_net_create.argtypes = [C.c_int, C.c_int, C.POINTER(LayerDesc)]
+_L.ftnn_net_destroy.restype = None
+_L.ftnn_net_destroy.argtypes = [_vp]
+_L.ftnn_net_output_elems.restype = C.c_int64
+_L.ftnn_net_output_elems.argtypes = [_vp]
+_L.ftnn_net_run.argtypes = [_vp, _vp, _vp, C.c_int, _vp]
+
+
+class Net:
+    """ftnn_net_*: a chain of conv layers with device-resident activations.
+    `layers` is a list of dicts with keys type, shape (C, IH, IW, KN, KW, KH, pad, stride),
+    threshold, alpha, qw (packed weights, int64 CUDA tensor, kept alive here)."""
+
+    def __init__(self, batch, layers):
+        self.batch = batch
+        self._weights = [l["qw"] for l in layers]
+        arr = (LayerDesc * len(layers))()
+        for d, l in zip(arr, layers):
+            c, ih, iw, kn, kw, kh, pad, stride = l["shape"]
+            d.type, d.C, d.H, d.W, d.KN, d.KH, d.KW, d.pad, d.stride = l["type"], c, ih, iw, kn, kh, kw, pad, stride
+            d.threshold, d.prelu_alpha, d.d_qw = l["threshold"], l["alpha"], _dev(l["qw"])
+        self._h = _L.ftnn_net_create(batch, len(layers), arr)
+        if not self._h:
+            raise FtnnError(_L.ftnn_last_error().decode())
+        c, ih, iw, kn, kw, kh, pad, stride = layers[-1]["shape"]
+        self.out_shape = (batch, kn, out_dim(ih, pad, kh, stride), out_dim(iw, pad, kw, stride))
+        assert int(_L.ftnn_net_output_elems(self._h)) == int(np.prod(self.out_shape))
+
+    def run(self, x, out=None, graph=False):
+        import torch
+        if out is None:
+            out = torch.empty(self.out_shape, dtype=torch.float32, device=x.device)
+        _check(_L.ftnn_net_run(self._h, _dev(x, torch.float32), _dev(out, torch.float32), int(graph), _stream()))
+        return out
+
+    def close(self):
+        if self._h:
+            _L.ftnn_net_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
 
 
 # -------------------------------------------------- reference (host) entry points

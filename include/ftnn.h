@@ -202,6 +202,36 @@ FTNN_API int ftnn_conv(int type, const float *d_x, const float *d_thr, const int
               int W_stride, float prelu_alpha, void *d_scratch, float *d_y, void *stream);
 
 /*
+ * A chain of conv layers with device-resident activations: the e2e mode of the reference's
+ * layer driver (src/timing_layers.c:182-207 feeds each layer's output to the next one), here
+ * without the host round trip per layer.  All device memory (two activation buffers, the
+ * quantiser scratch, per-layer threshold arrays) is allocated by ftnn_net_create; a run
+ * allocates nothing.  Packed weights stay the caller's and must outlive the net.
+ */
+typedef struct ftnn_layer {
+    int type;             /* TNN / TBN / BTN / BNN                               */
+    int C, H, W;          /* input channels, height, width                       */
+    int KN, KH, KW;       /* kernels, kernel height, kernel width                */
+    int pad, stride;      /* same in both directions, as the reference's tables  */
+    float threshold;      /* activation threshold, applied to every batch item   */
+    float prelu_alpha;
+    const int64_t *d_qw;  /* packed weights on the device (ftnn_pack_weights)    */
+} ftnn_layer_t;
+
+typedef struct ftnn_net ftnn_net_t;
+
+/* NULL on failure (ftnn_last_error() says why): every layer's input must be the previous
+ * layer's output shape */
+FTNN_API ftnn_net_t *ftnn_net_create(int batch, int n_layers, const ftnn_layer_t *layers);
+FTNN_API void ftnn_net_destroy(ftnn_net_t *net);
+/* elements of the final output (batch * KN * OH * OW of the last layer) */
+FTNN_API int64_t ftnn_net_output_elems(const ftnn_net_t *net);
+/* d_x: fp32 NCHW input of layer 0; d_y: fp32 NCHW output of the last layer.  use_graph != 0
+ * records the layer launches into a HIP graph on first use (and again whenever d_x, d_y or
+ * the stream change) and replays it afterwards. */
+FTNN_API int ftnn_net_run(ftnn_net_t *net, const float *d_x, float *d_y, int use_graph, void *stream);
+
+/*
  * Weight packers on the device: fp32 (KN,C,KH,KW) -> Packing-2 rows.  ternary != 0 is
  * ternarize_opt_avx2 (src/utils.c:468-521), ternary == 0 is binarize_opt_avx2
  * (src/utils.c:634-675).  d_thr[KN].

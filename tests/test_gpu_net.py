@@ -1,0 +1,83 @@
+"""The layer chain (ftnn_net_*): device-resident e2e mode of the reference's layer driver
+(src/timing_layers.c:182-207).  Bit-exact against the oracle run layer by layer; HIP-graph
+replays are checked one by one against the eager result with other work in between."""
+import numpy as np
+import pytest
+
+from fastertnn_amd import synth, TNN, TBN, BTN, BNN, act_is_ternary, weight_is_ternary
+
+pytestmark = pytest.mark.gpu
+
+# (type, (C, IH, IW, KN, KW, KH, pad, stride)): a shrunk ResNet-like stack with every network type
+STACK = [
+    (TNN, (3, 40, 40, 64, 7, 7, 3, 2)),
+    (TNN, (64, 20, 20, 64, 3, 3, 1, 2)),
+    (TNN, (64, 10, 10, 64, 3, 3, 1, 1)),
+    (TBN, (64, 10, 10, 128, 3, 3, 1, 2)),
+    (BTN, (128, 5, 5, 128, 3, 3, 1, 1)),
+    (BNN, (128, 5, 5, 192, 1, 1, 0, 1)),
+    (TNN, (192, 5, 5, 100, 1, 1, 0, 1)),
+]
+
+
+def build(hip, oracle, batch):
+    import torch
+    layers, host = [], []
+    for i, (typ, shape) in enumerate(STACK):
+        c, ih, iw, kn, kw, kh, pad, stride = shape
+        wt = weight_is_ternary(typ)
+        w = synth.ternary(600 + i, (kn, c, kh, kw)) if wt else synth.binary(600 + i, (kn, c, kh, kw))
+        wthr = np.full(kn, 0.5 if wt else 0.0, np.float32)
+        qw = oracle.pack_weights(w, wthr, wt)
+        thr = 0.5 if act_is_ternary(typ) else 0.0
+        host.append((typ, shape, qw, thr))
+        layers.append(dict(type=typ, shape=shape, threshold=thr, alpha=0.5, qw=torch.from_numpy(qw).cuda()))
+    return hip.Net(batch, layers), host
+
+
+def oracle_chain(oracle, host, x):
+    for typ, (c, ih, iw, kn, kw, kh, pad, stride), qw, thr in host:
+        x = oracle.conv(typ, x, np.full(x.shape[0], thr, np.float32), qw, kn, kh, kw, pad, stride, 0.5)
+    return x
+
+
+def test_chain_matches_the_oracle_layer_by_layer(hip, oracle):
+    import torch
+    batch = 3
+    net, host = build(hip, oracle, batch)
+    x = synth.normal(1, (batch, 3, 40, 40))
+    want = oracle_chain(oracle, host, x)
+    xd = torch.from_numpy(x).cuda()
+    got = net.run(xd)
+    assert got.cpu().numpy().tobytes() == want.tobytes()
+    # HIP graph: several replays, with eager work and synchronisation in between, each checked
+    s = torch.cuda.Stream()
+    out = torch.empty_like(got)
+    with torch.cuda.stream(s):
+        for rep in range(4):
+            out.fill_(-1.0)
+            net.run(xd, out=out, graph=True)
+            s.synchronize()
+            assert out.cpu().numpy().tobytes() == want.tobytes(), "replay %d" % rep
+            (torch.ones(1000, device="cuda") * rep).sum().item()
+        # new input contents in the same buffer: the recorded graph must see them
+        x2 = synth.normal(2, (batch, 3, 40, 40))
+        xd.copy_(torch.from_numpy(x2).cuda())
+        net.run(xd, out=out, graph=True)
+        s.synchronize()
+        assert out.cpu().numpy().tobytes() == oracle_chain(oracle, host, x2).tobytes()
+        # a different output buffer forces a new recording
+        out2 = torch.empty_like(out)
+        net.run(xd, out=out2, graph=True)
+        s.synchronize()
+        assert torch.equal(out, out2)
+    net.close()
+
+
+def test_chain_rejects_mismatched_layers(hip, oracle):
+    import torch
+    qw = torch.zeros(64 * 2 * 4, dtype=torch.int64, device="cuda")
+    good = dict(type=TNN, shape=(64, 8, 8, 64, 1, 1, 0, 1), threshold=0.5, alpha=0.5, qw=qw)
+    bad = dict(type=TNN, shape=(32, 8, 8, 64, 1, 1, 0, 1), threshold=0.5, alpha=0.5, qw=qw)
+    with pytest.raises(hip.FtnnError, match="not the output"):
+        hip.Net(2, [good, bad])
