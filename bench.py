@@ -107,7 +107,8 @@ def conv_latency(torch, lib, typ, shape, batch, seed, reps=20):
     wthr = torch.full((kn,), 0.5 if wt else 0.0, device="cuda")
     qw = lib.pack_weights(w, wthr, wt)
     oh, ow = lib.out_dim(ih, pad, kh, stride), lib.out_dim(iw, pad, kw, stride)
-    scratch = torch.empty(lib.pack_scratch_bytes(batch, c, ih, iw, at), dtype=torch.uint8, device="cuda")
+    scratch = torch.empty(lib.conv_scratch_bytes(typ, batch, c, ih, iw, kn, kh, kw, pad, stride), dtype=torch.uint8,
+                          device="cuda")
     y = torch.empty((batch, kn, oh, ow), device="cuda")
 
     def step():

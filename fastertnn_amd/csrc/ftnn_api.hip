@@ -176,6 +176,22 @@ int64_t ftnn_pack_scratch_bytes(int N, int C, int H, int W, int ternary) {
     return (int64_t)N * H * W * cpack_of(C) * (ternary ? 16 : 8);
 }
 
+int64_t ftnn_conv_scratch_bytes(int type, int N, int C, int H, int W, int KN, int KH, int KW, int H_pad,
+                                int W_pad, int H_stride, int W_stride) {
+    int OH, OW;
+    if (check_conv_shape(N, C, H, W, H_pad, W_pad, KH, KW, H_stride, W_stride, &OH, &OW) != FTNN_OK || KN <= 0)
+        return 0;
+    const bool at = (type == kTNN || type == kTBN), wt = (type == kTNN || type == kBTN);
+    int64_t bytes = ftnn_pack_scratch_bytes(N, C, H, W, at);
+    int T, Kd;
+    if (dense_applies(C, KH, KW, &T, &Kd)) {
+        bytes = (bytes + 255) / 256 * 256;
+        bytes += ((int64_t)N * OH * OW * round4(Kd) * (at ? 16 : 8) + 255) / 256 * 256;
+        bytes += (int64_t)KN * round4(Kd) * (wt ? 16 : 8);
+    }
+    return bytes;
+}
+
 int ftnn_quantize_im2row(int ternary, const float* d_x, const float* d_thr, int N, int C, int H,
                          int W, int H_pad, int W_pad, int kH, int kW, int H_stride, int W_stride,
                          int64_t* d_out, void* d_scratch, void* stream) {
@@ -320,6 +336,25 @@ int ftnn_conv(int type, const float* d_x, const float* d_thr, const int64_t* d_q
     const bool act_ternary = (type == kTNN || type == kTBN);
     hipError_t e = launch_quantize(act_ternary, d_x, d_thr, N, C, H, W, d_scratch, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "quantize launch");
+    int T, Kd;
+    if (dense_applies(C, KH, KW, &T, &Kd)) {
+        // few channels: re-pack both operands with several taps per word and run the plain GEMM
+        const bool w_ternary = (type == kTNN || type == kBTN);
+        char* base = static_cast<char*>(d_scratch);
+        const int64_t p_bytes = (ftnn_pack_scratch_bytes(N, C, H, W, act_ternary) + 255) / 256 * 256;
+        const int64_t rows_bytes =
+            ((int64_t)N * OH * OW * round4(Kd) * (act_ternary ? 16 : 8) + 255) / 256 * 256;
+        int64_t* d_rows = reinterpret_cast<int64_t*>(base + p_bytes);
+        int64_t* d_wd = reinterpret_cast<int64_t*>(base + p_bytes + rows_bytes);
+        e = launch_dense_rows(act_ternary, d_scratch, N, C, H, W, H_pad, W_pad, KH, KW, H_stride, W_stride,
+                              d_rows, (hipStream_t)stream);
+        if (e != hipSuccess) return hip_fail(e, "dense rows launch");
+        e = launch_dense_weights(w_ternary, d_qw, KN, C, KH, KW, d_wd, (hipStream_t)stream);
+        if (e != hipSuccess) return hip_fail(e, "dense weights launch");
+        e = launch_mm(type, d_rows, d_wd, (int64_t)N * OH * OW, OH * OW, KN, round4(Kd), C * KH * KW,
+                      prelu_alpha, d_y, (hipStream_t)stream);
+        return e == hipSuccess ? FTNN_OK : hip_fail(e, "mm launch");
+    }
     const ConvGeom cg = {H, W, cpack_of(C), OH, OW, KW, cpack_of(C) * KH * KW, H_pad, W_pad, H_stride, W_stride};
     e = launch_mm_implicit(type, d_scratch, d_qw, cg, N, KN, C * KH * KW, prelu_alpha, d_y, (hipStream_t)stream);
     return e == hipSuccess ? FTNN_OK : hip_fail(e, "implicit-im2row mm launch");
@@ -390,7 +425,8 @@ void tnns_conv(testcase_t* t) {
     float* d_thr = (float*)upload(SLOT_THR, t->input_thresholds, (size_t)N * sizeof(float));
     int64_t* d_w = (int64_t*)upload(SLOT_W, t->quantized_kernel_packing2,
                                     (size_t)KN * ftnn_row_words(C, KH, KW, w_tern) * sizeof(int64_t));
-    void* d_scr = dev_buf(SLOT_SCRATCH, (size_t)ftnn_pack_scratch_bytes(N, C, H, W, act_tern));
+    void* d_scr = dev_buf(SLOT_SCRATCH, (size_t)ftnn_conv_scratch_bytes(type, N, C, H, W, KN, KH, KW, t->paddingH,
+                                                                  t->paddingW, t->strideH, t->strideW));
     const size_t y_bytes = rows * KN * sizeof(float);
     float* d_y = (float*)dev_buf(SLOT_Y, y_bytes);
     if (ftnn_conv(type, d_x, d_thr, d_w, N, C, H, W, KN, KH, KW, t->paddingH, t->paddingW,

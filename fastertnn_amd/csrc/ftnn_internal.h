@@ -40,6 +40,13 @@ hipError_t launch_mm_implicit(int type, const void* d_p, const int64_t* d_b, con
 hipError_t launch_quantize(bool ternary, const float* d_x, const float* d_thr, int N, int C, int H, int W,
                            void* d_p, hipStream_t st);
 
+// dense re-packing of both operands for layers with C <= 32 (several taps per 64-lane word)
+bool dense_applies(int C, int KH, int KW, int* T_out, int* Kd_out);
+hipError_t launch_dense_rows(bool ternary, const void* d_p, int N, int C, int H, int W, int H_pad, int W_pad,
+                             int kH, int kW, int H_stride, int W_stride, int64_t* d_out, hipStream_t st);
+hipError_t launch_dense_weights(bool ternary, const int64_t* d_qw, int KN, int C, int kH, int kW,
+                                int64_t* d_out, hipStream_t st);
+
 // ---- mfma_kernels.hip: matrix-core formulation (int8 or fp4 operands expanded into d_scratch) ----
 int64_t mfma_fragment_bytes(bool f4, int64_t rows, int Kw);
 hipError_t launch_mfma_expand(bool f4, bool ternary, const int64_t* d_rows, int rows, int Kw, void* d_out,

@@ -84,7 +84,8 @@ ftnn_net_t* ftnn_net_create(int batch, int n_layers, const ftnn_layer_t* layers)
         net->OW.push_back(out_dim(L.W, L.pad, L.KW, L.stride));
         const int64_t out = (int64_t)batch * L.KN * net->OH[i] * net->OW[i];
         if (i < n_layers - 1 && out > max_act) max_act = out;
-        const int64_t scr = ftnn_pack_scratch_bytes(batch, L.C, L.H, L.W, L.type == kTNN || L.type == kTBN);
+        const int64_t scr = ftnn_conv_scratch_bytes(L.type, batch, L.C, L.H, L.W, L.KN, L.KH, L.KW, L.pad, L.pad,
+                                                    L.stride, L.stride);
         if (scr > max_scratch) max_scratch = scr;
         net->out_elems = out;
     }

@@ -205,7 +205,139 @@ __global__ __launch_bounds__(256) void k_pack_weights(const float* __restrict__ 
     }
 }
 
+// ------------------------------------------------------- dense rows for small C
+// With C <= 32 a Packing-2 word carries C live lanes out of 64 (C = 3 in an RGB stem: 3 of 64).
+// The GEMM result only depends on the multiset of (activation lane, weight lane) pairs, so both
+// operands may be re-packed with T = 64 / C taps per word: lane (tap t, channel c) -> word t / T,
+// bit (t % T) * C + c.  Unused lanes are (sign 0, zero 1) / 0 exactly like the reference's fill, and
+// the existing GEMM kernels run unchanged on Kd = ceil(KH*KW / T) words instead of KH*KW.
+
+// activations: one work-item per (row, dense word); gathers T taps from P (C_pack = 1)
+template <bool TERN>
+__global__ __launch_bounds__(256) void k_dense_rows(const unsigned long long* __restrict__ P, int C, int T,
+                                                    int H, int W, int OH, int OW, int KW, int taps, int Kd,
+                                                    int Kdw, int H_pad, int W_pad, int H_stride,
+                                                    int W_stride, int64_t total,
+                                                    unsigned long long* __restrict__ out) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= total) return;
+    const int64_t r = e / Kdw;
+    const int d = (int)(e - r * Kdw);
+    unsigned long long s = 0ull, z = ~0ull;
+    if (d < Kd) {
+        const int ow = (int)(r % OW);
+        const int64_t t2 = r / OW;
+        const int oh = (int)(t2 % OH);
+        const int64_t n = t2 / OH;
+        const unsigned long long cmask = (1ull << C) - 1ull;
+        for (int j = 0; j < T; j++) {
+            const int tap = d * T + j;
+            if (tap >= taps) break;
+            const int kh = tap / KW, kw = tap - kh * KW;
+            const int ih = oh * H_stride + kh - H_pad, iw = ow * W_stride + kw - W_pad;
+            if (ih >= 0 && ih < H && iw >= 0 && iw < W) {
+                const size_t o = (size_t)n * H * W + (size_t)ih * W + iw;
+                if (TERN) {
+                    const ulonglong2 v = reinterpret_cast<const ulonglong2*>(P)[o];
+                    s |= (v.x & cmask) << (j * C);
+                    z &= ~((~v.y & cmask) << (j * C));
+                } else {
+                    s |= (P[o] & cmask) << (j * C);
+                }
+            }
+        }
+    }
+    if (!TERN && d >= Kd) s = 0ull;
+    if (TERN) {
+        unsigned long long* row = out + (size_t)r * 2 * Kdw;
+        row[p2_pos(d, 0)] = s;
+        row[p2_pos(d, 1)] = z;
+    } else {
+        out[(size_t)r * Kdw + d] = s;
+    }
+}
+
+// weights: one work-item per (kernel, dense word); source rows are the reference's packed rows
+// with C_pack = 1 (word index = tap)
+template <bool TERN>
+__global__ __launch_bounds__(256) void k_dense_weights(const unsigned long long* __restrict__ Q, int C, int T,
+                                                       int taps, int Kw, int Kd, int Kdw, int64_t total,
+                                                       unsigned long long* __restrict__ out) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= total) return;
+    const int64_t n = e / Kdw;
+    const int d = (int)(e - n * Kdw);
+    unsigned long long s = 0ull, z = TERN ? ~0ull : 0ull;
+    if (d < Kd) {
+        const unsigned long long cmask = (1ull << C) - 1ull;
+        for (int j = 0; j < T; j++) {
+            const int tap = d * T + j;
+            if (tap >= taps) break;
+            if (TERN) {
+                const unsigned long long* row = Q + (size_t)n * 2 * Kw;
+                s |= (row[p2_pos(tap, 0)] & cmask) << (j * C);
+                z &= ~((~row[p2_pos(tap, 1)] & cmask) << (j * C));
+            } else {
+                s |= (Q[(size_t)n * Kw + tap] & cmask) << (j * C);
+            }
+        }
+    }
+    if (TERN) {
+        unsigned long long* row = out + (size_t)n * 2 * Kdw;
+        row[p2_pos(d, 0)] = s;
+        row[p2_pos(d, 1)] = z;
+    } else {
+        out[(size_t)n * Kdw + d] = s;
+    }
+}
+
 }  // namespace
+
+bool dense_applies(int C, int KH, int KW, int* T_out, int* Kd_out) {
+    if (C > 32) return false;
+    const int T = 64 / C, taps = KH * KW;
+    const int Kd = (taps + T - 1) / T;
+    if (T_out) *T_out = T;
+    if (Kd_out) *Kd_out = Kd;
+    return round4(taps) >= 2 * round4(Kd);   // at least halves the GEMM work
+}
+
+hipError_t launch_dense_rows(bool ternary, const void* d_p, int N, int C, int H, int W, int H_pad, int W_pad,
+                             int kH, int kW, int H_stride, int W_stride, int64_t* d_out, hipStream_t st) {
+    int T, Kd;
+    dense_applies(C, kH, kW, &T, &Kd);
+    const int OH = out_dim(H, H_pad, kH, H_stride), OW = out_dim(W, W_pad, kW, W_stride);
+    const int Kdw = round4(Kd);
+    const int64_t total = (int64_t)N * OH * OW * Kdw;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    const unsigned long long* P = static_cast<const unsigned long long*>(d_p);
+    unsigned long long* out = reinterpret_cast<unsigned long long*>(d_out);
+    if (ternary)
+        hipLaunchKernelGGL((k_dense_rows<true>), dim3(blocks), dim3(256), 0, st, P, C, T, H, W, OH, OW, kW,
+                           kH * kW, Kd, Kdw, H_pad, W_pad, H_stride, W_stride, total, out);
+    else
+        hipLaunchKernelGGL((k_dense_rows<false>), dim3(blocks), dim3(256), 0, st, P, C, T, H, W, OH, OW, kW,
+                           kH * kW, Kd, Kdw, H_pad, W_pad, H_stride, W_stride, total, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_dense_weights(bool ternary, const int64_t* d_qw, int KN, int C, int kH, int kW,
+                                int64_t* d_out, hipStream_t st) {
+    int T, Kd;
+    dense_applies(C, kH, kW, &T, &Kd);
+    const int Kw = round4(kH * kW), Kdw = round4(Kd);
+    const int64_t total = (int64_t)KN * Kdw;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    const unsigned long long* Q = reinterpret_cast<const unsigned long long*>(d_qw);
+    unsigned long long* out = reinterpret_cast<unsigned long long*>(d_out);
+    if (ternary)
+        hipLaunchKernelGGL((k_dense_weights<true>), dim3(blocks), dim3(256), 0, st, Q, C, T, kH * kW, Kw, Kd, Kdw,
+                           total, out);
+    else
+        hipLaunchKernelGGL((k_dense_weights<false>), dim3(blocks), dim3(256), 0, st, Q, C, T, kH * kW, Kw, Kd,
+                           Kdw, total, out);
+    return hipGetLastError();
+}
 
 hipError_t launch_quantize(bool ternary, const float* d_x, const float* d_thr, int N, int C, int H, int W,
                            void* d_p, hipStream_t st) {

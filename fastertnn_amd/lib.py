@@ -39,6 +39,8 @@ _L.ftnn_expand_bytes.restype = C.c_int64
 _L.ftnn_expand_bytes.argtypes = [C.c_int] * 3
 _L.ftnn_expand_rows.argtypes = [C.c_int, C.c_int, _vp, C.c_int, C.c_int, _vp, _vp]
 _L.ftnn_mm_expanded.argtypes = [C.c_int, C.c_int, _vp, _vp] + [C.c_int] * 6 + [C.c_float, _vp, _vp]
+_L.ftnn_conv_scratch_bytes.restype = C.c_int64
+_L.ftnn_conv_scratch_bytes.argtypes = [C.c_int] * 12
 _L.ftnn_conv.argtypes = [C.c_int, _vp, _vp, _vp] + [C.c_int] * 11 + [C.c_float, _vp, _vp, _vp]
 _L.ftnn_pack_weights.argtypes = [C.c_int, _vp, _vp] + [C.c_int] * 4 + [_vp, _vp]
 _L.ftnn_pack_gemm_operand.argtypes = [_vp, C.c_int, C.c_int, _vp, _vp]
@@ -58,7 +60,7 @@ EXPORTS = ("tnns_conv", "tnns_gemm", "t2r_p2_opt", "b2r", "mm_tnn", "mm_tbn", "m
            "ftnn_pack_scratch_bytes", "ftnn_quantize_im2row", "ftnn_mm", "ftnn_conv",
            "ftnn_pack_weights", "ftnn_pack_gemm_operand", "ftnn_select_engine", "ftnn_mm_scratch_bytes",
            "ftnn_mm_engine", "ftnn_expand_bytes", "ftnn_expand_rows", "ftnn_mm_expanded",
-           "ftnn_net_create", "ftnn_net_destroy", "ftnn_net_output_elems", "ftnn_net_run")
+           "ftnn_conv_scratch_bytes", "ftnn_net_create", "ftnn_net_destroy", "ftnn_net_output_elems", "ftnn_net_run")
 
 ENGINE_AUTO, ENGINE_VALU, ENGINE_MFMA_I8, ENGINE_MFMA_F4 = 0, 1, 2, 3
 ENGINE_NAMES = {ENGINE_VALU: "valu", ENGINE_MFMA_I8: "mfma_i8", ENGINE_MFMA_F4: "mfma_f4"}
@@ -132,6 +134,10 @@ def mm(typ, a, b, n, oh, ow, kn, k, alpha, k_unpack=0, out=None):
     return out
 
 
+def conv_scratch_bytes(typ, n, c, h, w, kn, kh, kw, pad, stride):
+    return int(_L.ftnn_conv_scratch_bytes(typ, n, c, h, w, kn, kh, kw, pad, pad, stride, stride))
+
+
 def select_engine(typ, n, oh, ow, kn, k):
     return int(_L.ftnn_select_engine(typ, n, oh, ow, kn, k))
 
@@ -183,7 +189,8 @@ def conv(typ, x, thr, qw, kn, kh, kw, pad, stride, alpha, scratch=None, out=None
         raise FtnnError("kernel larger than padded input")
     tern = act_is_ternary(typ)
     if scratch is None:
-        scratch = torch.empty(pack_scratch_bytes(n, c, h, w, tern), dtype=torch.uint8, device=x.device)
+        scratch = torch.empty(conv_scratch_bytes(typ, n, c, h, w, kn, kh, kw, pad, stride), dtype=torch.uint8,
+                              device=x.device)
     if out is None:
         out = torch.empty((n, kn, oh, ow), dtype=torch.float32, device=x.device)
     _check(_L.ftnn_conv(typ, _dev(x, torch.float32), _dev(thr, torch.float32), _dev(qw), n, c, h, w, kn, kh,

@@ -193,10 +193,14 @@ FTNN_API int ftnn_mm_expanded(int engine, int type, const void *d_a_exp, const v
 
 /*
  * One conv layer on the device (src/tnns/tnns_cpu_mm_p2.c:6-80): the input is quantised
- * once into d_scratch (ftnn_pack_scratch_bytes() bytes) and the GEMM gathers its im2row
- * operand from there, so the im2row matrix of t2r_p2_opt / b2r is never written to memory.
- * Same result as ftnn_quantize_im2row followed by ftnn_mm.
+ * once into d_scratch (ftnn_conv_scratch_bytes() bytes, 16-byte aligned) and the GEMM gathers
+ * its im2row operand from there, so the im2row matrix of t2r_p2_opt / b2r is never written to
+ * memory.  Layers with C <= 32 re-pack both operands with several kernel taps per 64-lane word
+ * first (an RGB stem uses 3 of 64 lanes otherwise).  Same result as ftnn_quantize_im2row
+ * followed by ftnn_mm.
  */
+FTNN_API int64_t ftnn_conv_scratch_bytes(int type, int N, int C, int H, int W, int KN, int KH, int KW,
+                                int H_pad, int W_pad, int H_stride, int W_stride);
 FTNN_API int ftnn_conv(int type, const float *d_x, const float *d_thr, const int64_t *d_qw, int N, int C,
               int H, int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride,
               int W_stride, float prelu_alpha, void *d_scratch, float *d_y, void *stream);

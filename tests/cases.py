@@ -34,6 +34,12 @@ EXTRA_SHAPES = [
     (70, 9, 5, 33, 2, 4, 2, 3),
     (200, 1, 1, 10, 1, 1, 0, 1),
     (64, 4, 4, 7, 6, 6, 1, 1),
+    # few channels: several kernel taps share a 64-lane word in the device's dense re-packing
+    (8, 9, 9, 12, 3, 3, 1, 1),
+    (16, 11, 7, 40, 5, 5, 2, 2),
+    (1, 6, 6, 3, 3, 3, 1, 1),
+    (21, 8, 8, 9, 3, 3, 0, 1),
+    (20, 16, 16, 33, 7, 7, 3, 2),
 ]
 
 ALL_TYPES = (TNN, TBN, BTN, BNN)
