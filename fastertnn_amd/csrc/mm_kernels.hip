@@ -24,6 +24,7 @@
 //     distinct banks.
 // A workgroup is 4 wavefronts sharing one A tile of 64*TM rows; wavefront w
 // computes columns [w*TN, (w+1)*TN) of the workgroup's 4*TN columns.
+#include <stdio.h>
 #include <stdlib.h>
 
 #include "ftnn_internal.h"
@@ -341,10 +342,15 @@ hipError_t launch_mode(const uint32_t* A, const uint32_t* B, float* Y, int64_t M
     auto wgs = [&](int tm, int tn) {
         return ((M + 64 * tm - 1) / (64 * tm)) * ((KN + 4 * tn - 1) / (4 * tn));
     };
-    static const char* force = getenv("FTNN_MM_TILE");   // tuning aid: "28", "14" or "12" forces a tile
-    if (force && force[0] == '2') return launch_cfg<MODE, 2, 8, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
-    if (force && force[1] == '4') return launch_cfg<MODE, 1, 4, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
-    if (force && force[1] == '2') return launch_cfg<MODE, 1, 2, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+    static const char* force = getenv("FTNN_MM_TILE");   // tuning aid: "TM,TN" forces a tile
+    if (force) {
+        int tm = 0, tn = 0;
+        sscanf(force, "%d,%d", &tm, &tn);
+#define FTNN_TRY(TM_, TN_) \
+    if (tm == TM_ && tn == TN_) return launch_cfg<MODE, TM_, TN_, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+        FTNN_TRY(2, 8) FTNN_TRY(1, 4) FTNN_TRY(1, 2) FTNN_TRY(1, 8) FTNN_TRY(1, 16) FTNN_TRY(2, 4) FTNN_TRY(2, 16)
+#undef FTNN_TRY
+    }
     if (wgs(2, 8) >= 3072) return launch_cfg<MODE, 2, 8, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
     if (wgs(1, 4) >= 2048) return launch_cfg<MODE, 1, 4, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
     return launch_cfg<MODE, 1, 2, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
