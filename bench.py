@@ -193,7 +193,7 @@ def main():
     args = parse()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported "
-                 "(the path shards over output rows with no exchange, see DESIGN.md)" % args.gpus)
+                 "(the path would shard over output rows with no exchange)" % args.gpus)
     import numpy as np
     import torch
     if not torch.cuda.is_available():
