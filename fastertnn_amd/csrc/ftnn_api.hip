@@ -2,6 +2,8 @@
 // the reference's host-memory entry points built on top of them.
 #include <stdarg.h>
 #include <stdio.h>
+
+#include <mutex>
 #include <stdlib.h>
 #include <string.h>
 
@@ -48,6 +50,9 @@ struct HostCtx {
     size_t cap[6] = {0, 0, 0, 0, 0, 0};
 };
 static HostCtx g_ctx;
+// The reference's entry points are called from one thread (its drivers are single-threaded); the
+// workspace is nevertheless guarded so that concurrent callers serialise instead of racing.
+static std::mutex g_ctx_mutex;
 
 [[noreturn]] static void die(const char* what) {
     // the reference reports failure by abort() (src/timing_layers.c:156-159)
@@ -114,6 +119,7 @@ enum { SLOT_X = 0, SLOT_THR, SLOT_W, SLOT_ROWS, SLOT_SCRATCH, SLOT_Y };
 static int64_t* host_quantize_im2row(bool ternary, float* x, float* thr, int N, int C, int H, int W,
                                      int H_pad, int W_pad, int kH, int kW, int H_stride,
                                      int W_stride) {
+    std::lock_guard<std::mutex> lock(g_ctx_mutex);
     int OH, OW;
     if (check_conv_shape(N, C, H, W, H_pad, W_pad, kH, kW, H_stride, W_stride, &OH, &OW) != FTNN_OK)
         die(ternary ? "t2r_p2_opt" : "b2r");
@@ -133,6 +139,7 @@ static int64_t* host_quantize_im2row(bool ternary, float* x, float* thr, int N, 
 
 static float* host_mm(int type, int64_t* a, int64_t* b, int N, int OH, int OW, int KN, int K,
                       int K_unpack, float alpha) {
+    std::lock_guard<std::mutex> lock(g_ctx_mutex);
     if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0) {
         fail(FTNN_EINVAL, "non-positive GEMM dimension");
         die("mm");
@@ -355,7 +362,8 @@ int ftnn_conv(int type, const float* d_x, const float* d_thr, const int64_t* d_q
                       prelu_alpha, d_y, (hipStream_t)stream);
         return e == hipSuccess ? FTNN_OK : hip_fail(e, "mm launch");
     }
-    const ConvGeom cg = {H, W, cpack_of(C), OH, OW, KW, cpack_of(C) * KH * KW, H_pad, W_pad, H_stride, W_stride};
+    const ConvGeom cg = {H, W, cpack_of(C), OH, OW, KW, cpack_of(C) * KH * KW, H_pad, W_pad, H_stride, W_stride,
+                         make_fastdiv((uint32_t)OW), make_fastdiv((uint32_t)cpack_of(C)), make_fastdiv((uint32_t)KW)};
     e = launch_mm_implicit(type, d_scratch, d_qw, cg, N, KN, C * KH * KW, prelu_alpha, d_y, (hipStream_t)stream);
     return e == hipSuccess ? FTNN_OK : hip_fail(e, "implicit-im2row mm launch");
 }
@@ -408,6 +416,7 @@ float* mm_bnn(int64_t* a, int64_t* b, int N, int OH, int OW, int KN, int K, int 
 }
 
 void tnns_conv(testcase_t* t) {
+    std::lock_guard<std::mutex> lock(g_ctx_mutex);
     const int type = (int)t->type;
     const int N = t->batchcount, C = t->channelcount, H = t->inputH, W = t->inputW;
     const int KN = t->kernelcount, KH = t->kernelH, KW = t->kernelW;

@@ -11,10 +11,29 @@ inline int cpack_of(int C) { return (C + 63) / 64; }
 inline int round4(int k) { return 4 * ((k + 3) / 4); }
 inline int out_dim(int in, int pad, int k, int stride) { return (in + 2 * pad - k) / stride + 1; }
 
+// Division of a 32-bit unsigned n by a fixed d without the ~25-instruction expansion of "/":
+// m = floor(2^32 / d) (saturated for d = 1) under-estimates the quotient by at most one, which one
+// compare fixes.  Exact for every n < 2^32, d >= 1.
+struct FastDiv {
+    uint32_t d, m;
+};
+inline FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f;
+    f.d = d;
+    f.m = d <= 1 ? 0xffffffffu : (uint32_t)((1ull << 32) / d);
+    return f;
+}
+__device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDiv& f) {
+    uint32_t q = __umulhi(n, f.m);
+    if (n - q * f.d >= f.d) q++;
+    return q;
+}
+
 // geometry of one conv layer as the implicit-im2row GEMM needs it
 struct ConvGeom {
     int H, W, CP, OH, OW, KW, K;   // K = C_pack*KH*KW words per plane before rounding
     int H_pad, W_pad, H_stride, W_stride;
+    FastDiv dOW, dCP, dKW;
 };
 
 // record a failure text for ftnn_last_error(); returns `code`

@@ -275,13 +275,10 @@ template <bool F4, bool SWAP>
 hipError_t launch_gemm(const uint4* Pf, const uint4* Qf, float* Y, int M, int KN, int OHW, int KB,
                        int bias, int form, float alpha, hipStream_t st) {
     auto kern = k_mfma<F4, SWAP>;
-    static bool configured = false;   // the opt-in to more than 64 KiB of dynamic LDS is per kernel
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
-        if (e != hipSuccess) return e;
-        configured = true;
-    }
+    // the opt-in to more than 64 KiB of dynamic LDS is per kernel; done once, thread-safe
+    static const hipError_t configured = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
+    if (configured != hipSuccess) return configured;
     const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN;
     dim3 grid((prow + 255) / 256, (qrow + 255) / 256);
     if (grid.y > 65535) return hipErrorInvalidValue;

@@ -107,7 +107,7 @@ template <int MODE, int TM, int TN, int GC, bool IMPL>
 __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
                                             const uint32_t* __restrict__ B,
                                             float* __restrict__ Y, int M, int KN, int OHW, int G,
-                                            int K_unpack, float alpha, ConvGeom cg) {
+                                            int K_unpack, float alpha, FastDiv dOHW, ConvGeom cg) {
     using T = Traits<MODE>;
     constexpr int BM = 64 * TM;
     constexpr int AG = T::kAGroup, BG = T::kBGroup;
@@ -162,9 +162,9 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
 #pragma unroll
         for (int it = 0; it < ITI; it++) {
             const uint32_t r = (uint32_t)min(row0 + sr + it * 64, (int64_t)M - 1);
-            const uint32_t n = r / (uint32_t)OHW;
+            const uint32_t n = fastdiv(r, dOHW);
             const uint32_t pix = r - n * (uint32_t)OHW;
-            const int oh = (int)(pix / (uint32_t)cg.OW), ow = (int)pix - oh * cg.OW;
+            const int oh = (int)fastdiv(pix, cg.dOW), ow = (int)pix - oh * cg.OW;
             ih0[it] = oh * cg.H_stride - cg.H_pad;
             iw0[it] = ow * cg.W_stride - cg.W_pad;
             pix0[it] = (size_t)n * cg.H * cg.W;
@@ -178,9 +178,9 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
     // chunk without divisions (chunks are fetched in order, one group each)
     int f_ic = 0, f_kh = 0, f_kw = 0;
     if (IMPL) {
-        const int tap = sq / cg.CP;
+        const int tap = (int)fastdiv((uint32_t)sq, cg.dCP);
         f_ic = sq - tap * cg.CP;
-        f_kh = tap / cg.KW;
+        f_kh = (int)fastdiv((uint32_t)tap, cg.dKW);
         f_kw = tap - f_kh * cg.KW;
     }
     // issue the global loads of group-chunk starting at group g0 into the staging registers
@@ -189,9 +189,10 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
             const bool valid = g0 * 4 + sq < cg.K;
             const int ic = f_ic, kh = f_kh, kw = f_kw;
             f_ic += 4;
+            const int wraps = cg.CP >= 4 ? 1 : 4;   // uniform: one wrap suffices when C_pack >= 4
 #pragma unroll
-            for (int w = 0; w < 4; w++) {   // at most 4 wraps (C_pack = 1); one when C_pack >= 4
-                if (f_ic >= cg.CP) {
+            for (int w = 0; w < 4; w++) {
+                if (w < wraps && f_ic >= cg.CP) {
                     f_ic -= cg.CP;
                     if (++f_kw == cg.KW) {
                         f_kw = 0;
@@ -295,7 +296,7 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
     for (int a = 0; a < TM; a++) {
         const int64_t i = row0 + lane + 64 * a;
         if (i < M) {
-            const uint32_t img = (uint32_t)i / (uint32_t)OHW;
+            const uint32_t img = fastdiv((uint32_t)i, dOHW);
             const uint32_t pix = (uint32_t)i - img * (uint32_t)OHW;
 #pragma unroll
             for (int b = 0; b < TN; b++) {
@@ -329,7 +330,7 @@ hipError_t launch_cfg(const uint32_t* A, const uint32_t* B, float* Y, int64_t M,
     const int64_t gy = (KN + 4 * TN - 1) / (4 * TN);
     if (gx > 0x7fffffffLL || gy > 65535) return hipErrorInvalidValue;
     hipLaunchKernelGGL((k_mm<MODE, TM, TN, GC, IMPL>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
-                       A, B, Y, (int)M, KN, OHW, G, K_unpack, alpha, cg);
+                       A, B, Y, (int)M, KN, OHW, G, K_unpack, alpha, make_fastdiv((uint32_t)OHW), cg);
     return hipGetLastError();
 }
 
