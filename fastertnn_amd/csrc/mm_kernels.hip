@@ -349,10 +349,11 @@ hipError_t launch_mode(const uint32_t* A, const uint32_t* B, float* Y, int64_t M
         sscanf(force, "%d,%d", &tm, &tn);
 #define FTNN_TRY(TM_, TN_) \
     if (tm == TM_ && tn == TN_) return launch_cfg<MODE, TM_, TN_, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
-        FTNN_TRY(2, 8) FTNN_TRY(1, 4) FTNN_TRY(1, 2) FTNN_TRY(1, 8) FTNN_TRY(1, 16) FTNN_TRY(2, 4) FTNN_TRY(2, 16)
+        FTNN_TRY(2, 8) FTNN_TRY(1, 8) FTNN_TRY(1, 4) FTNN_TRY(1, 2)
 #undef FTNN_TRY
     }
     if (wgs(2, 8) >= 3072) return launch_cfg<MODE, 2, 8, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+    if (wgs(1, 8) >= 1536) return launch_cfg<MODE, 1, 8, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
     if (wgs(1, 4) >= 2048) return launch_cfg<MODE, 1, 4, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
     return launch_cfg<MODE, 1, 2, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
 }
