@@ -292,31 +292,44 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
     }
 
     const int lanes_total = G * 4 * 64;  // 64 * Kw
+    // PReLU in the reference's form for the type, from the integer accumulators of (row a, column b)
+    auto finish = [&](int a, int b) -> float {
+        if (MODE == kTNN) {
+            // src/tnns/mm_p2_final_tnn_avx2.c:178,204-208
+            const int acc = lanes_total - (int)(cz[a][b] + 2u * cn[a][b]);
+            float f = (float)acc;
+            if (f <= 0) f *= alpha;
+            return f;
+        }
+        int r;
+        if (MODE == kTBN) r = lanes_total - (int)rowz[a] - 2 * (int)cn[a][b];
+        else if (MODE == kBTN) r = lanes_total - (int)colz[b] - 2 * (int)cn[a][b];
+        else r = K_unpack - 2 * (int)cn[a][b];
+        // src/tnns/mm_p2_final_tbn_avx2.c:72-73
+        return r >= 0 ? (float)r : alpha * r;
+    };
+    // Row-major result (OHW == 1, the GEMM entry points): a lane's TN columns are contiguous, so they
+    // leave as 16-byte stores (full 32-byte sectors) instead of TN scattered dwords.
+    const bool vec = TN % 4 == 0 && OHW == 1 && (KN & 3) == 0 && col0 + TN <= KN &&
+                     (reinterpret_cast<uintptr_t>(Y) & 15u) == 0;
 #pragma unroll
     for (int a = 0; a < TM; a++) {
         const int64_t i = row0 + lane + 64 * a;
         if (i < M) {
-            const uint32_t img = fastdiv((uint32_t)i, dOHW);
-            const uint32_t pix = (uint32_t)i - img * (uint32_t)OHW;
+            if (vec) {
+                float* yr = Y + (size_t)i * KN + col0;
 #pragma unroll
-            for (int b = 0; b < TN; b++) {
-                const int j = col0 + b;
-                if (j < KN) {
-                    float f;
-                    if (MODE == kTNN) {
-                        // src/tnns/mm_p2_final_tnn_avx2.c:178,204-208
-                        const int acc = lanes_total - (int)(cz[a][b] + 2u * cn[a][b]);
-                        f = (float)acc;
-                        if (f <= 0) f *= alpha;
-                    } else {
-                        int r;
-                        if (MODE == kTBN) r = lanes_total - (int)rowz[a] - 2 * (int)cn[a][b];
-                        else if (MODE == kBTN) r = lanes_total - (int)colz[b] - 2 * (int)cn[a][b];
-                        else r = K_unpack - 2 * (int)cn[a][b];
-                        // src/tnns/mm_p2_final_tbn_avx2.c:72-73
-                        f = r >= 0 ? (float)r : alpha * r;
-                    }
-                    Y[((size_t)img * KN + j) * OHW + pix] = f;
+                for (int b4 = 0; b4 < TN / 4; b4++)
+                    *reinterpret_cast<float4*>(yr + 4 * b4) =
+                        make_float4(finish(a, 4 * b4), finish(a, 4 * b4 + 1), finish(a, 4 * b4 + 2),
+                                    finish(a, 4 * b4 + 3));
+            } else {
+                const uint32_t img = fastdiv((uint32_t)i, dOHW);
+                const uint32_t pix = (uint32_t)i - img * (uint32_t)OHW;
+#pragma unroll
+                for (int b = 0; b < TN; b++) {
+                    const int j = col0 + b;
+                    if (j < KN) Y[((size_t)img * KN + j) * OHW + pix] = finish(a, b);
                 }
             }
         }
