@@ -231,11 +231,14 @@ int ftnn_mm(int type, const int64_t* d_a, const int64_t* d_b, int N, int OH, int
 }
 
 // Engine choice by shape, from measurements on MI355X: the matrix-core path works on 256 x 256
-// tiles and pays two expansion passes, so it needs a few hundred tiles of real work to win.
+// tiles and pays two expansion passes (about 25 us of fixed cost), the vector-ALU kernel runs near
+// 0.3 PMAC/s.  fp4 wins from about 1.2e10 lane-MACs on, provided there are enough tiles to spread
+// over the CUs; below that the vector-ALU kernel is faster.
 static int select_engine(int type, int64_t M, int KN, int Kw) {
     (void)type;
     const int64_t tiles = ((M + 255) / 256) * ((KN + 255) / 256);
-    if (tiles >= 128 && KN >= 256 && Kw >= 16 && 64LL * Kw < (1LL << 24)) return FTNN_ENGINE_MFMA_F4;
+    const double lane_macs = (double)M * KN * 64.0 * Kw;
+    if (lane_macs >= 1.2e10 && tiles >= 48 && KN >= 128 && 64LL * Kw < (1LL << 24)) return FTNN_ENGINE_MFMA_F4;
     return FTNN_ENGINE_VALU;
 }
 

@@ -82,6 +82,28 @@ def test_bad_arguments_are_rejected_without_touching_the_device():
     assert L.ftnn_pack_weights(1, p, p, 0, 8, 3, 3, p, None) == -1
 
 
+def test_engine_selection_and_scratch_sizes_need_no_device():
+    import fastertnn_amd.lib as lib
+    # the large GEMM goes to the fp4 matrix-core engine, layer-sized problems stay on the vector ALU
+    assert lib.select_engine(0, 8192, 1, 1, 8192, 512) == lib.ENGINE_MFMA_F4
+    assert lib.select_engine(0, 2048, 1, 1, 2048, 256) == lib.ENGINE_MFMA_F4
+    assert lib.select_engine(0, 1, 56, 56, 256, 36) == lib.ENGINE_VALU
+    assert lib.select_engine(0, 32, 56, 56, 64, 9) == lib.ENGINE_VALU
+    assert lib.select_engine(0, 512, 1, 1, 512, 512) == lib.ENGINE_VALU          # too few tiles
+    # fp32 accumulation of fp4 products is exact only below 2^24 lanes: never chosen beyond
+    assert lib.select_engine(0, 4096, 1, 1, 4096, 1 << 18) == lib.ENGINE_VALU
+    assert lib.mm_scratch_bytes(lib.ENGINE_VALU, 0, 8192, 1, 1, 8192, 512) == 0
+    assert lib.mm_scratch_bytes(lib.ENGINE_MFMA_F4, 0, 8192, 1, 1, 8192, 512) == 2 * 256 * 512 * 1024
+    assert lib.mm_scratch_bytes(lib.ENGINE_MFMA_I8, 0, 33, 1, 1, 1, 4) == (2 + 1) * 8 * 1024
+    assert lib.mm_scratch_bytes(lib.ENGINE_AUTO, 0, 8192, 1, 1, 8192, 512) == 2 * 256 * 512 * 1024
+    assert lib._L.ftnn_expand_bytes(lib.ENGINE_MFMA_F4, 100, 6) == 4 * 8 * 1024
+    assert lib._L.ftnn_expand_bytes(lib.ENGINE_VALU, 100, 6) == 0
+    # conv scratch: the quantised input, plus dense rows and weights when C <= 32 packs several taps per word
+    assert lib.conv_scratch_bytes(0, 2, 64, 8, 8, 16, 3, 3, 1, 1) == lib.pack_scratch_bytes(2, 64, 8, 8, 1)
+    dense = lib.conv_scratch_bytes(0, 2, 3, 32, 32, 16, 7, 7, 3, 2)
+    assert dense == 2 * 32 * 32 * 16 + 2 * 16 * 16 * 4 * 16 + 16 * 4 * 16
+
+
 def test_missing_library_is_an_import_error(tmp_path):
     """no silent CPU fallback: the binding refuses to import without the built library"""
     pkg = tmp_path / "fastertnn_amd"
