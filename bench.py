@@ -135,6 +135,17 @@ def conv_latency(torch, lib, typ, shape, batch, seed, reps=20):
         yr = ref.conv(typ, xh, thrh, qwh, kn, kh, kw, pad, stride, 0.5)
         out["cpu_ms"] = round((time.perf_counter() - t0) * 1e3, 2)
         out["bit_exact_vs_reference"] = bool(np.ascontiguousarray(yh).tobytes() == yr.tobytes())
+    # the reference's "baseline" (Packing 0) build beside its "final" one, as its Makefile pairs them
+    if O.ReferenceBaseline.available():
+        base = O.ReferenceBaseline()
+        qw0 = base.pack_weights(w.cpu().numpy(), wthr.cpu().numpy(), wt)
+        try:
+            t0 = time.perf_counter()
+            yb = base.conv(typ, xh, thrh, qw0, kn, kh, kw, pad, stride, 0.5)
+            out["cpu_reference_baseline_build_ms"] = round((time.perf_counter() - t0) * 1e3, 1)
+            out["bit_exact_vs_reference_baseline_build"] = bool(np.ascontiguousarray(yh).tobytes() == yb.tobytes())
+        finally:
+            base.free_weights(qw0)
     return out
 
 

@@ -1,12 +1,14 @@
 """ctypes bindings of the checker: TEST INFRASTRUCTURE ONLY.
 
-Two libraries are bound here:
+Three libraries are bound here:
 
 * ``Oracle``     -- ``libftnn_oracle.so``, the plain-C restatement in this directory.
 * ``Reference``  -- ``_ref/libref_final.so``, the reference's own AVX2 "final" path
   compiled from its sources (present only where ``make ref`` ran or its output
   was carried along).  It validates the restatement, writes the golden vectors
   and serves as the CPU baseline of the benchmark.
+* ``ReferenceBaseline`` -- ``_ref/libref_baseline.so``, the reference's Packing-0
+  "baseline" build (src/tnns/tnns_cpu_naive.c), an independent second reference.
 
 Only the test-suite, the smoke check and the benchmark's CPU-baseline leg may
 import this module; the shipped library never does.
@@ -20,6 +22,7 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 ORACLE_SO = os.path.join(HERE, "libftnn_oracle.so")
 REF_SO = os.path.join(HERE, "_ref", "libref_final.so")
+REF_BASELINE_SO = os.path.join(HERE, "_ref", "libref_baseline.so")
 
 TNN, TBN, BTN, BNN = 0, 1, 2, 3
 TYPE_NAMES = {TNN: "tnn", TBN: "tbn", BTN: "btn", BNN: "bnn"}
@@ -236,3 +239,54 @@ class Reference:
         self.libc.free(px)
         oh, ow = out_dim(h, pad, kh, stride), out_dim(wd, pad, kw, stride)
         return self._take(y, n * kn * oh * ow, np.float32).reshape(n, kn, oh, ow)
+
+
+class ReferenceBaseline:
+    """The reference's "baseline" build (Packing 0, separate ternarise / img2row / popcount GEMM /
+    PReLU passes, src/tnns/tnns_cpu_naive.c:255-292): an implementation independent of the Packing-2
+    path, used as a second reference and for the reference's own "baseline vs final" comparison
+    (Makefile:50)."""
+
+    def __init__(self, path=REF_BASELINE_SO):
+        if not os.path.exists(path):
+            raise FileNotFoundError(path)
+        L = self.lib = C.CDLL(path)
+        self.libc = C.CDLL(None)
+        self.libc.free.argtypes = [C.c_void_p]
+        L.ternarize_naive.restype = C.c_void_p
+        L.binarize_naive.restype = C.c_void_p
+        L.tnns_conv.restype = None
+
+    @staticmethod
+    def available():
+        return os.path.exists(REF_BASELINE_SO)
+
+    def pack_weights(self, w, wthr, ternary):
+        """ternarize_naive / binarize_naive on the weights, as src/timing_layers.c:129-133 does;
+        returns the raw pointer (freed by free_weights)"""
+        w = _f32(w)
+        wthr = _f32(wthr)
+        kn, c, kh, kw = w.shape
+        fn = self.lib.ternarize_naive if ternary else self.lib.binarize_naive
+        ptr = fn(_p(w, _f32p), _p(wthr, _f32p), kn, c, kh, kw, 0, 0)
+        if not ptr:
+            raise MemoryError("reference returned NULL")
+        return ptr
+
+    def free_weights(self, ptr):
+        self.libc.free(ptr)
+
+    def conv(self, typ, x, thr, qw0_ptr, kn, kh, kw, pad, stride, alpha):
+        x = aligned_copy(_f32(x))
+        thr = _f32(thr)
+        n, c, h, w = x.shape
+        t = _Testcase(type=typ, batchcount=n, channelcount=c, inputW=w, inputH=h, kernelcount=kn,
+                      kernelW=kw, kernelH=kh, paddingW=pad, paddingH=pad, strideW=stride, strideH=stride,
+                      preluAlpha=alpha, input_thresholds=thr.ctypes.data, input=x.ctypes.data,
+                      quantized_kernel_packing0=qw0_ptr)
+        self.lib.tnns_conv(C.byref(t))
+        oh, ow = out_dim(h, pad, kh, stride), out_dim(w, pad, kw, stride)
+        buf = (C.c_char * (n * kn * oh * ow * 4)).from_address(t.output)
+        out = np.frombuffer(buf, dtype=np.float32).copy().reshape(n, kn, oh, ow)
+        self.libc.free(t.output)
+        return out

@@ -27,6 +27,14 @@ def reference():
 
 
 @pytest.fixture(scope="session")
+def reference_baseline():
+    from oracle.ftnn_oracle import ReferenceBaseline
+    if not ReferenceBaseline.available():
+        pytest.skip("compiled reference baseline (oracle/_ref) not present")
+    return ReferenceBaseline()
+
+
+@pytest.fixture(scope="session")
 def hip():
     """The HIP library binding; fails (does not skip) when the library is missing."""
     import torch

@@ -61,3 +61,23 @@ def test_negative_alpha_and_alpha_one(hip, oracle):
             want = oracle.conv(typ, L["x"], L["thr"], qw, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], alpha)
             got = hip.host_conv(typ, L["x"], L["thr"], qw, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], alpha)
             assert got.tobytes() == want.tobytes(), (TYPE_NAMES[typ], alpha)
+
+
+@pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
+def test_hip_layer_equals_the_reference_baseline_build(hip, oracle, reference_baseline, typ):
+    """second reference: the Packing-0 "baseline" build (src/tnns/tnns_cpu_naive.c:255-292), which shares
+    no kernel code with the Packing-2 path the library replaces"""
+    at, wt = act_is_ternary(typ), weight_is_ternary(typ)
+    shapes = REF_TEST_SHAPES + EXTRA_SHAPES
+    for si in (1, 2, 5, 6, 9, 10, 12, 13, 18, 22):
+        L = make_layer(typ, shapes[si], 4, seed=2500 + si)
+        print("case", TYPE_NAMES[typ], shapes[si], flush=True)
+        qw0 = reference_baseline.pack_weights(L["w"], L["wthr"], wt)
+        try:
+            want = reference_baseline.conv(typ, L["x"], L["thr"], qw0, L["kn"], L["kh"], L["kw"], L["pad"],
+                                           L["stride"], L["alpha"])
+        finally:
+            reference_baseline.free_weights(qw0)
+        qw2 = oracle.pack_weights(L["w"], L["wthr"], wt)
+        got = hip.host_conv(typ, L["x"], L["thr"], qw2, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], L["alpha"])
+        assert got.tobytes() == want.tobytes()

@@ -55,3 +55,22 @@ def test_gemm_operands_and_tnns_gemm(oracle, reference):
         bo, br = oracle.pack_gemm_operand(b), reference.pack_gemm_operand(b)
         assert np.array_equal(ao, ar) and np.array_equal(bo, br)
         assert oracle.gemm(ao, bo, m, n, p // 64).tobytes() == reference.mm(TNN, ar, br, m, 1, 1, n, p // 64, 1.0).tobytes()
+
+
+@pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
+def test_independent_baseline_pipeline_agrees(oracle, reference_baseline, typ):
+    """the reference's Packing-0 "baseline" build (ternarise -> img2row -> popcount GEMM -> PReLU as
+    four passes, src/tnns/tnns_cpu_naive.c:255-292) shares no kernel code with the Packing-2 path;
+    its layer output must equal the oracle's bit for bit"""
+    at, wt = act_is_ternary(typ), weight_is_ternary(typ)
+    for si in (0, 1, 2, 4, 5, 6, 9, 10, 12, 13, 18, 20):
+        L = make_layer(typ, SHAPES[si], 4, seed=900 + si)
+        qw0 = reference_baseline.pack_weights(L["w"], L["wthr"], wt)
+        try:
+            want = reference_baseline.conv(typ, L["x"], L["thr"], qw0, L["kn"], L["kh"], L["kw"], L["pad"],
+                                           L["stride"], L["alpha"])
+        finally:
+            reference_baseline.free_weights(qw0)
+        got = oracle.conv(typ, L["x"], L["thr"], oracle.pack_weights(L["w"], L["wthr"], wt), L["kn"], L["kh"],
+                          L["kw"], L["pad"], L["stride"], L["alpha"])
+        assert got.tobytes() == want.tobytes(), SHAPES[si]
