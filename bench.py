@@ -90,6 +90,80 @@ def cpu_gemm_baseline(a_host, b_host, rows, n, kw, alpha):
     return y, dt, kind
 
 
+def small_gemm(torch, lib, m, n, k, reps=30):
+    """the reference's own CPU-runnable GEMM case on every engine (whole call, HIP events), the
+    host entry point mm_tnn (host pointers in and out) and the CPU reference on one core"""
+    import numpy as np
+    from fastertnn_amd import TNN
+    from oracle import ftnn_oracle as O
+    kw, alpha = k // 64, 0.5
+    a = ternary_operand(torch, lib, m, k, seed=1)
+    b = ternary_operand(torch, lib, n, k, seed=7)
+    y = torch.empty((m, n, 1, 1), dtype=torch.float32, device="cuda")
+    scratch = torch.empty(max(lib.mm_scratch_bytes(e, TNN, m, 1, 1, n, kw) for e in lib.ENGINE_NAMES) or 16,
+                          dtype=torch.uint8, device="cuda")
+    a_h, b_h = O.aligned_copy(a.cpu().numpy()), O.aligned_copy(b.cpu().numpy())
+    cpu = O.Reference() if O.Reference.available() else O.Oracle()
+    t_cpu = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        want = cpu.mm(TNN, a_h, b_h, m, 1, 1, n, kw, alpha)
+        t_cpu.append(time.perf_counter() - t0)
+    out = {"cpu_ms": round(min(t_cpu) * 1e3, 3), "cpu_gmacs": round(float(m) * n * k / min(t_cpu) / 1e9, 1),
+           "auto_engine": lib.ENGINE_NAMES[lib.select_engine(TNN, m, 1, 1, n, kw)]}
+    for eng, name in lib.ENGINE_NAMES.items():
+        def run(eng=eng):
+            lib.mm_engine(eng, TNN, a, b, m, 1, 1, n, kw, alpha, out=y, scratch=scratch)
+        run()
+        t = event_times(torch, run, reps)
+        t = sum(t) / len(t)
+        out[name] = {"call_ms": round(t, 4), "gmacs": round(float(m) * n * k / t / 1e6, 1),
+                     "bit_exact_vs_cpu": bool(y.cpu().numpy().tobytes() == np.ascontiguousarray(want).tobytes())}
+    t_abi = []
+    for _ in range(10):
+        t0 = time.perf_counter()
+        got = lib.host_mm(TNN, a_h, b_h, m, 1, 1, n, kw, alpha)
+        t_abi.append(time.perf_counter() - t0)
+    out["abi_ms"] = round(min(t_abi) * 1e3, 3)
+    out["abi_bit_exact_vs_cpu"] = bool(got.tobytes() == np.ascontiguousarray(want).tobytes())
+    return out
+
+
+def other_types(torch, lib, a_tern, b_tern, m, n, k, reps=5):
+    """TBN / BTN / BNN on the headline shape: every engine's whole call and the vector-ALU kernel's
+    fraction of its roofline (2 lane-ops per dword pair for these types); binary operands are
+    uniform random words"""
+    from fastertnn_amd import TBN, BTN, BNN, act_is_ternary, weight_is_ternary
+    kw = k // 64
+    g = torch.Generator(device="cuda")
+    g.manual_seed(9)
+    a_bin = torch.randint(-2 ** 62, 2 ** 62, (m * kw,), generator=g, device="cuda", dtype=torch.int64)
+    b_bin = torch.randint(-2 ** 62, 2 ** 62, (n * kw,), generator=g, device="cuda", dtype=torch.int64)
+    y = torch.empty((m, n, 1, 1), dtype=torch.float32, device="cuda")
+    out = {}
+    for typ, name in ((TBN, "tbn"), (BTN, "btn"), (BNN, "bnn")):
+        a = a_tern if act_is_ternary(typ) else a_bin
+        b = b_tern if weight_is_ternary(typ) else b_bin
+        scratch = torch.empty(max(lib.mm_scratch_bytes(e, typ, m, 1, 1, n, kw) for e in lib.ENGINE_NAMES) or 16,
+                              dtype=torch.uint8, device="cuda")
+        row, first = {}, None
+        for eng, en in lib.ENGINE_NAMES.items():
+            def run(eng=eng):
+                lib.mm_engine(eng, typ, a, b, m, 1, 1, n, kw, 0.5, k if typ == BNN else 0, out=y, scratch=scratch)
+            run()
+            torch.cuda.synchronize()
+            if first is None:
+                first = y.clone()
+            same = bool(torch.equal(first, y))
+            t = event_times(torch, run, reps)
+            t = sum(t) / len(t)
+            row[en] = {"call_ms": round(t, 4), "gmacs": round(float(m) * n * k / t / 1e6, 1), "same_bits_as_valu": same}
+        row["valu_roofline_frac"] = round(2.0 * m * n * 2 * kw / (row["valu"]["call_ms"] * 1e-3) / 1e12 / VALU_PEAK_TOPS, 4)
+        out[name] = row
+        del scratch, first
+    return out
+
+
 def conv_latency(torch, lib, typ, shape, batch, seed, reps=20):
     """kernel-only (device buffers, HIP events) and ABI-inclusive (host pointers) latency"""
     import numpy as np
@@ -316,6 +390,8 @@ def main():
     extra = None
     if not args.no_extra:
         extra = {
+            "other_types_same_gemm_shape": other_types(torch, lib, a, b, m, n, k),
+            "tnn_gemm_256x256x4096": small_gemm(torch, lib, 256, 256, 4096),
             "tnn_conv_b1_c256_56x56_k3": conv_latency(torch, lib, TNN, (256, 56, 56, 256, 3, 3, 1, 1), 1, 2),
             "tbn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, TBN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 3),
             "btn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, BTN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 4),

@@ -103,7 +103,9 @@ __device__ __forceinline__ uint32_t popc4(const uint4& v) {
 // (n, oh, ow) from pixel (oh*s + kh - p, ow*s + kw - p) and applies the reference's fill rules
 // (src/tnns/ternarize2row_avx2.c:438-472, :748-755; src/tnns/binarize2row_avx2.c:151), so the
 // im2row matrix is never written to memory.
-template <int MODE, int TM, int TN, int GC, bool IMPL>
+// TR = true stores the result transposed, Y[column * M + row] (row-major GEMM results only): the
+// launcher uses it to run a BTN GEMM as a TBN GEMM with the operands exchanged, see launch_mm.
+template <int MODE, int TM, int TN, int GC, bool IMPL, bool TR = false>
 __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
                                             const uint32_t* __restrict__ B,
                                             float* __restrict__ Y, int M, int KN, int OHW, int G,
@@ -316,7 +318,13 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
     for (int a = 0; a < TM; a++) {
         const int64_t i = row0 + lane + 64 * a;
         if (i < M) {
-            if (vec) {
+            if (TR) {   // consecutive lanes write consecutive floats of one output row
+#pragma unroll
+                for (int b = 0; b < TN; b++) {
+                    const int j = col0 + b;
+                    if (j < KN) Y[(size_t)j * M + i] = finish(a, b);
+                }
+            } else if (vec) {
                 float* yr = Y + (size_t)i * KN + col0;
 #pragma unroll
                 for (int b4 = 0; b4 < TN / 4; b4++)
@@ -336,18 +344,18 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
     }
 }
 
-template <int MODE, int TM, int TN, int GC, bool IMPL>
+template <int MODE, int TM, int TN, int GC, bool IMPL, bool TR>
 hipError_t launch_cfg(const uint32_t* A, const uint32_t* B, float* Y, int64_t M, int KN, int OHW,
                       int G, int K_unpack, float alpha, const ConvGeom& cg, hipStream_t st) {
     const int64_t gx = (M + 64 * TM - 1) / (64 * TM);
     const int64_t gy = (KN + 4 * TN - 1) / (4 * TN);
     if (gx > 0x7fffffffLL || gy > 65535) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((k_mm<MODE, TM, TN, GC, IMPL>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
+    hipLaunchKernelGGL((k_mm<MODE, TM, TN, GC, IMPL, TR>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
                        A, B, Y, (int)M, KN, OHW, G, K_unpack, alpha, make_fastdiv((uint32_t)OHW), cg);
     return hipGetLastError();
 }
 
-template <int MODE, bool IMPL>
+template <int MODE, bool IMPL, bool TR = false>
 hipError_t launch_mode(const uint32_t* A, const uint32_t* B, float* Y, int64_t M, int KN, int OHW,
                        int G, int K_unpack, float alpha, const ConvGeom& cg, hipStream_t st) {
     // Tile choice (measured on MI355X): 128 x 32 tiles once they give each of the 256 CUs
@@ -361,14 +369,14 @@ hipError_t launch_mode(const uint32_t* A, const uint32_t* B, float* Y, int64_t M
         int tm = 0, tn = 0;
         sscanf(force, "%d,%d", &tm, &tn);
 #define FTNN_TRY(TM_, TN_) \
-    if (tm == TM_ && tn == TN_) return launch_cfg<MODE, TM_, TN_, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+    if (tm == TM_ && tn == TN_) return launch_cfg<MODE, TM_, TN_, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
         FTNN_TRY(2, 8) FTNN_TRY(1, 8) FTNN_TRY(1, 4) FTNN_TRY(1, 2)
 #undef FTNN_TRY
     }
-    if (wgs(2, 8) >= 3072) return launch_cfg<MODE, 2, 8, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
-    if (wgs(1, 8) >= 1536) return launch_cfg<MODE, 1, 8, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
-    if (wgs(1, 4) >= 2048) return launch_cfg<MODE, 1, 4, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
-    return launch_cfg<MODE, 1, 2, 1, IMPL>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+    if (wgs(2, 8) >= 3072) return launch_cfg<MODE, 2, 8, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+    if (wgs(1, 8) >= 1536) return launch_cfg<MODE, 1, 8, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+    if (wgs(1, 4) >= 2048) return launch_cfg<MODE, 1, 4, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+    return launch_cfg<MODE, 1, 2, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
 }
 
 }  // namespace
@@ -379,6 +387,14 @@ hipError_t launch_mm(int type, const int64_t* d_a, const int64_t* d_b, int64_t M
     const uint32_t* B = reinterpret_cast<const uint32_t*>(d_b);
     const int G = Kw / 4;
     const ConvGeom cg = {};
+    // A BTN product needs both planes of B next to a plane of A: (a ^ sb) & ~zb.  With B in scalar
+    // registers that is two scalar operands in one vector instruction, which the ISA does not
+    // encode, so the kernel pays a register copy per dword.  For a row-major result the same sums
+    // come from the TBN form with the operands exchanged (ternary B along the lanes, binary A in
+    // scalar registers) and the result stored transposed; both types share one PReLU form
+    // (src/tnns/mm_p2_final_tbn_avx2.c:72-73, src/tnns/mm_p2_final_btn_avx2.c:72-73).
+    if (type == kBTN && OHW == 1 && KN >= 64 && M <= 0x7fffffff)
+        return launch_mode<kTBN, false, true>(B, A, d_y, KN, (int)M, 1, G, K_unpack, alpha, cg, st);
     switch (type) {
         case kTNN: return launch_mode<kTNN, false>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
         case kTBN: return launch_mode<kTBN, false>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);

@@ -53,6 +53,27 @@ def test_engines_on_gemm_operands(hip, oracle, mnp):
         assert got.tobytes() == want.tobytes(), "engine %d" % eng
 
 
+@pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
+@pytest.mark.parametrize("mnk", [(1, 64, 4), (5, 65, 8), (70, 100, 12), (200, 257, 36), (1000, 64, 4),
+                                 (129, 1000, 8), (64, 63, 4), (300, 2048, 20)])
+def test_row_major_gemm_all_types(hip, oracle, typ, mnk):
+    """fully connected / GEMM-shaped results (OH = OW = 1) on random packed words, every type and
+    engine; a BTN product of this shape runs as the TBN form with the operands exchanged and a
+    transposed store, which ragged row and column counts on either side exercise"""
+    m, n, kw = mnk
+    rng = np.random.default_rng(1000 * typ + m + n + kw)
+    at, wt = act_is_ternary(typ), weight_is_ternary(typ)
+    a = rng.integers(-2 ** 63, 2 ** 63, size=m * kw * (2 if at else 1), dtype=np.int64)
+    b = rng.integers(-2 ** 63, 2 ** 63, size=n * kw * (2 if wt else 1), dtype=np.int64)
+    ku = 64 * kw - 7
+    a_d, b_d = _dev(a), _dev(b)
+    for alpha in (0.5, -0.25):
+        want = oracle.mm(typ, a, b, m, 1, 1, n, kw, alpha, ku)
+        for eng in (hip.ENGINE_VALU, hip.ENGINE_MFMA_I8, hip.ENGINE_MFMA_F4, hip.ENGINE_AUTO):
+            got = hip.mm_engine(eng, typ, a_d, b_d, m, 1, 1, n, kw, alpha, ku).cpu().numpy()
+            assert got.tobytes() == want.tobytes(), "engine %d alpha %g" % (eng, alpha)
+
+
 def test_lanes_flagged_zero_and_negative_count_as_zero(hip, oracle):
     """a lane with both its sign and its zero bit set is zero in the reference's formula
     (za|zb masks it); the expanded operands must agree"""
