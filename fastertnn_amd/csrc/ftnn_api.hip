@@ -162,6 +162,20 @@ static float* host_mm(int type, int64_t* a, int64_t* b, int N, int OH, int OW, i
     return y;
 }
 
+// the matrix-core layer with the weights already expanded (d_wf); d_p4 takes the quantised input
+int conv_f4_expanded(int type, const float* d_x, const float* d_thr, const void* d_wf, int N, int C, int H,
+                           int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride, int W_stride,
+                           float prelu_alpha, void* d_p4, float* d_y, hipStream_t st) {
+    const int OH = out_dim(H, H_pad, KH, H_stride), OW = out_dim(W, W_pad, KW, W_stride);
+    const bool act_ternary = (type == kTNN || type == kTBN);
+    hipError_t e = launch_quantize_f4(act_ternary, d_x, d_thr, N, C, H, W, d_p4, st);
+    if (e != hipSuccess) return hip_fail(e, "fp4 quantize launch");
+    const ConvGeom cg = {H, W, cpack_of(C), OH, OW, KW, cpack_of(C) * KH * KW, H_pad, W_pad, H_stride, W_stride,
+                         make_fastdiv((uint32_t)OW), make_fastdiv((uint32_t)cpack_of(C)), make_fastdiv((uint32_t)KW)};
+    e = launch_conv_f4(type, d_p4, d_wf, cg, N, KN, C * KH * KW, prelu_alpha, d_y, st);
+    return e == hipSuccess ? FTNN_OK : hip_fail(e, "fp4 conv launch");
+}
+
 }  // namespace ftnn
 
 using namespace ftnn;
@@ -183,6 +197,30 @@ int64_t ftnn_pack_scratch_bytes(int N, int C, int H, int W, int ternary) {
     return (int64_t)N * H * W * cpack_of(C) * (ternary ? 16 : 8);
 }
 
+// bytes of the two regions of the matrix-core layer path: P4 (32 bytes per pixel and 64 channels),
+// then the fp4 fragments of the weights
+static int64_t conv_f4_p4_bytes(int N, int C, int H, int W) {
+    return ((int64_t)N * H * W * cpack_of(C) * 32 + 255) / 256 * 256;
+}
+
+// Layer engine by shape, from measurements on MI355X: the fp4 matrix-core kernel wins wherever it
+// applies except on the few-channel layers that the dense re-packing shrinks.
+static int select_conv_engine(int type, int N, int C, int H, int W, int KN, int KH, int KW, int OH, int OW) {
+    (void)type; (void)N; (void)H; (void)W; (void)KN; (void)OH; (void)OW;
+    int T, Kd;
+    if (dense_applies(C, KH, KW, &T, &Kd)) return FTNN_ENGINE_VALU;
+    if (64LL * cpack_of(C) * KH * KW >= (1LL << 24)) return FTNN_ENGINE_VALU;   // fp32 accumulation must stay exact
+    return FTNN_ENGINE_MFMA_F4;
+}
+
+int ftnn_select_conv_engine(int type, int N, int C, int H, int W, int KN, int KH, int KW, int H_pad, int W_pad,
+                            int H_stride, int W_stride) {
+    int OH, OW;
+    if (check_conv_shape(N, C, H, W, H_pad, W_pad, KH, KW, H_stride, W_stride, &OH, &OW) != FTNN_OK || KN <= 0)
+        return FTNN_ENGINE_VALU;
+    return select_conv_engine(type, N, C, H, W, KN, KH, KW, OH, OW);
+}
+
 int64_t ftnn_conv_scratch_bytes(int type, int N, int C, int H, int W, int KN, int KH, int KW, int H_pad,
                                 int W_pad, int H_stride, int W_stride) {
     int OH, OW;
@@ -196,7 +234,9 @@ int64_t ftnn_conv_scratch_bytes(int type, int N, int C, int H, int W, int KN, in
         bytes += ((int64_t)N * OH * OW * round4(Kd) * (at ? 16 : 8) + 255) / 256 * 256;
         bytes += (int64_t)KN * round4(Kd) * (wt ? 16 : 8);
     }
-    return bytes;
+    // enough for either engine, so that one buffer serves ftnn_conv and ftnn_conv_engine
+    const int64_t f4 = conv_f4_p4_bytes(N, C, H, W) + mfma_fragment_bytes(true, KN, round4(cpack_of(C) * KH * KW));
+    return bytes > f4 ? bytes : f4;
 }
 
 int ftnn_quantize_im2row(int ternary, const float* d_x, const float* d_thr, int N, int C, int H,
@@ -331,9 +371,9 @@ int ftnn_mm_engine(int engine, int type, const int64_t* d_a, const int64_t* d_b,
     return e == hipSuccess ? FTNN_OK : hip_fail(e, "mfma mm launch");
 }
 
-int ftnn_conv(int type, const float* d_x, const float* d_thr, const int64_t* d_qw, int N, int C,
-              int H, int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride, int W_stride,
-              float prelu_alpha, void* d_scratch, float* d_y, void* stream) {
+int ftnn_conv_engine(int engine, int type, const float* d_x, const float* d_thr, const int64_t* d_qw, int N,
+                     int C, int H, int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride,
+                     int W_stride, float prelu_alpha, void* d_scratch, float* d_y, void* stream) {
     if (type < kTNN || type > kBNN) return fail(FTNN_EINVAL, "unknown network type %d", type);
     int OH, OW;
     int rc = check_conv_shape(N, C, H, W, H_pad, W_pad, KH, KW, H_stride, W_stride, &OH, &OW);
@@ -343,13 +383,27 @@ int ftnn_conv(int type, const float* d_x, const float* d_thr, const int64_t* d_q
     if (!aligned16(d_scratch) || !aligned16(d_qw))
         return fail(FTNN_EINVAL, "d_scratch and d_qw must be 16-byte aligned");
     if ((int64_t)N * OH * OW > 0x7fffffffLL) return fail(FTNN_EINVAL, "more than 2^31-1 output rows");
+    if (engine == FTNN_ENGINE_AUTO) engine = select_conv_engine(type, N, C, H, W, KN, KH, KW, OH, OW);
     const bool act_ternary = (type == kTNN || type == kTBN);
+    const bool w_ternary = (type == kTNN || type == kBTN);
+    if (engine == FTNN_ENGINE_MFMA_F4) {
+        const int Kw = round4(cpack_of(C) * KH * KW);
+        if (64LL * Kw >= (1LL << 24))
+            return fail(FTNN_EINVAL, "K too long for exact fp32 accumulation; use the vector-ALU engine");
+        if ((int64_t)N * H * W * cpack_of(C) > 0x7fffffffLL)
+            return fail(FTNN_EINVAL, "more than 2^31-1 input pixel words");
+        void* d_wf = static_cast<char*>(d_scratch) + conv_f4_p4_bytes(N, C, H, W);
+        hipError_t e = launch_mfma_expand(true, w_ternary, d_qw, KN, Kw, d_wf, (hipStream_t)stream);
+        if (e != hipSuccess) return hip_fail(e, "weight expansion launch");
+        return conv_f4_expanded(type, d_x, d_thr, d_wf, N, C, H, W, KN, KH, KW, H_pad, W_pad, H_stride, W_stride,
+                                prelu_alpha, d_scratch, d_y, (hipStream_t)stream);
+    }
+    if (engine != FTNN_ENGINE_VALU) return fail(FTNN_EINVAL, "layer engine %d (vector ALU and fp4 only)", engine);
     hipError_t e = launch_quantize(act_ternary, d_x, d_thr, N, C, H, W, d_scratch, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "quantize launch");
     int T, Kd;
     if (dense_applies(C, KH, KW, &T, &Kd)) {
         // few channels: re-pack both operands with several taps per word and run the plain GEMM
-        const bool w_ternary = (type == kTNN || type == kBTN);
         char* base = static_cast<char*>(d_scratch);
         const int64_t p_bytes = (ftnn_pack_scratch_bytes(N, C, H, W, act_ternary) + 255) / 256 * 256;
         const int64_t rows_bytes =
@@ -369,6 +423,13 @@ int ftnn_conv(int type, const float* d_x, const float* d_thr, const int64_t* d_q
                          make_fastdiv((uint32_t)OW), make_fastdiv((uint32_t)cpack_of(C)), make_fastdiv((uint32_t)KW)};
     e = launch_mm_implicit(type, d_scratch, d_qw, cg, N, KN, C * KH * KW, prelu_alpha, d_y, (hipStream_t)stream);
     return e == hipSuccess ? FTNN_OK : hip_fail(e, "implicit-im2row mm launch");
+}
+
+int ftnn_conv(int type, const float* d_x, const float* d_thr, const int64_t* d_qw, int N, int C,
+              int H, int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride, int W_stride,
+              float prelu_alpha, void* d_scratch, float* d_y, void* stream) {
+    return ftnn_conv_engine(FTNN_ENGINE_AUTO, type, d_x, d_thr, d_qw, N, C, H, W, KN, KH, KW, H_pad, W_pad,
+                            H_stride, W_stride, prelu_alpha, d_scratch, d_y, stream);
 }
 
 int ftnn_pack_weights(int ternary, const float* d_w, const float* d_thr, int KN, int C, int KH,

@@ -59,6 +59,10 @@ hipError_t launch_mm_implicit(int type, const void* d_p, const int64_t* d_b, con
 hipError_t launch_quantize(bool ternary, const float* d_x, const float* d_thr, int N, int C, int H, int W,
                            void* d_p, hipStream_t st);
 
+// quantise only, into fp4 nibbles: fp32 NCHW -> P4[n][C_pack][pixel][32 bytes] (operand of launch_conv_f4)
+hipError_t launch_quantize_f4(bool ternary, const float* d_x, const float* d_thr, int N, int C, int H, int W,
+                              void* d_p4, hipStream_t st);
+
 // dense re-packing of both operands for layers with C <= 32 (several taps per 64-lane word)
 bool dense_applies(int C, int KH, int KW, int* T_out, int* Kd_out);
 hipError_t launch_dense_rows(bool ternary, const void* d_p, int N, int C, int H, int W, int H_pad, int W_pad,
@@ -75,5 +79,18 @@ hipError_t launch_mfma_gemm(bool f4, int type, const void* d_af, const void* d_b
 hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* d_b, int64_t M, int OHW,
                           int KN, int Kw, int K_unpack, float alpha, float* d_y, void* d_scratch,
                           hipStream_t st);
+
+// conv layer on the fp4 matrix cores: activations from launch_quantize_f4, weights as the fp4 fragments
+// launch_mfma_expand(true, ...) makes of the packed weight rows (Kw = round4(cg.K) words per row)
+hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const ConvGeom& cg, int N, int KN,
+                          int K_unpack, float alpha, float* d_y, hipStream_t st);
+
+
+// ---- ftnn_api.hip ----
+// the fp4 layer with weights expanded beforehand (d_wf: launch_mfma_expand(true, ...) of the packed rows);
+// d_p4 receives the quantised input: N*H*W*C_pack*32 bytes.  Arguments already validated.
+int conv_f4_expanded(int type, const float* d_x, const float* d_thr, const void* d_wf, int N, int C, int H,
+                     int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride, int W_stride,
+                     float prelu_alpha, void* d_p4, float* d_y, hipStream_t st);
 
 }  // namespace ftnn

@@ -11,6 +11,7 @@ struct ftnn_net {
     std::vector<ftnn_layer_t> layers;
     std::vector<int> OH, OW;
     std::vector<float*> d_thr;       // per layer: batch copies of its threshold
+    std::vector<void*> d_wf;         // per layer on the fp4 engine: its weights as matrix-core fragments
     float* d_act[2] = {nullptr, nullptr};
     void* d_scratch = nullptr;
     int64_t out_elems = 0;
@@ -31,8 +32,14 @@ int enqueue_layers(ftnn_net* net, const float* d_x, float* d_y, hipStream_t st) 
     for (int i = 0; i < n; i++) {
         const ftnn_layer_t& L = net->layers[i];
         float* out = (i == n - 1) ? d_y : net->d_act[i & 1];
-        int rc = ftnn_conv(L.type, in, net->d_thr[i], L.d_qw, net->batch, L.C, L.H, L.W, L.KN, L.KH, L.KW, L.pad,
-                           L.pad, L.stride, L.stride, L.prelu_alpha, net->d_scratch, out, st);
+        int rc;
+        if (net->d_wf[i])
+            rc = conv_f4_expanded(L.type, in, net->d_thr[i], net->d_wf[i], net->batch, L.C, L.H, L.W, L.KN, L.KH,
+                                  L.KW, L.pad, L.pad, L.stride, L.stride, L.prelu_alpha, net->d_scratch, out, st);
+        else
+            rc = ftnn_conv_engine(FTNN_ENGINE_VALU, L.type, in, net->d_thr[i], L.d_qw, net->batch, L.C, L.H, L.W,
+                                  L.KN, L.KH, L.KW, L.pad, L.pad, L.stride, L.stride, L.prelu_alpha,
+                                  net->d_scratch, out, st);
         if (rc != FTNN_OK) return rc;
         in = out;
     }
@@ -101,6 +108,20 @@ ftnn_net_t* ftnn_net_create(int batch, int n_layers, const ftnn_layer_t* layers)
         for (int b = 0; b < batch; b++) host[(size_t)b] = layers[i].threshold;
         good = hipMemcpy(d, host.data(), (size_t)batch * sizeof(float), hipMemcpyHostToDevice) == hipSuccess;
     }
+    // layers that run on the fp4 matrix cores get their weights expanded once, here
+    net->d_wf.assign((size_t)n_layers, nullptr);
+    for (int i = 0; i < n_layers && good; i++) {
+        const ftnn_layer_t& L = layers[i];
+        if (ftnn_select_conv_engine(L.type, batch, L.C, L.H, L.W, L.KN, L.KH, L.KW, L.pad, L.pad, L.stride,
+                                    L.stride) != FTNN_ENGINE_MFMA_F4)
+            continue;
+        const int Kw = round4(cpack_of(L.C) * L.KH * L.KW);
+        good = hipMalloc(&net->d_wf[i], (size_t)mfma_fragment_bytes(true, L.KN, Kw)) == hipSuccess;
+        if (!good) break;
+        good = launch_mfma_expand(true, L.type == kTNN || L.type == kBTN, L.d_qw, L.KN, Kw, net->d_wf[i], nullptr) ==
+                   hipSuccess &&
+               hipStreamSynchronize(nullptr) == hipSuccess;
+    }
     if (!good) {
         fail(FTNN_ENOMEM, "device allocation for the layer chain failed");
         ftnn_net_destroy(net);
@@ -113,6 +134,8 @@ void ftnn_net_destroy(ftnn_net_t* net) {
     if (!net) return;
     drop_graph(net);
     for (float* p : net->d_thr) (void)hipFree(p);
+    for (void* p : net->d_wf)
+        if (p) (void)hipFree(p);
     for (int b = 0; b < 2; b++)
         if (net->d_act[b]) (void)hipFree(net->d_act[b]);
     if (net->d_scratch) (void)hipFree(net->d_scratch);

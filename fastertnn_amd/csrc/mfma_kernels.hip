@@ -271,6 +271,203 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
         }
 }
 
+// ------------------------------------------------------------ conv layer (fp4)
+// Layer-sized problems (a few GMAC, 10^3..10^5 output pixels) are latency-, not throughput-bound,
+// and their im2row operand does not exist in memory.  This kernel therefore works on small tiles
+// with many wavefronts in flight and gathers its activation fragments itself:
+//   * a wavefront owns 64 kernels x 64 output pixels (2 x 2 MFMA blocks, 64 accumulator
+//     registers).  A workgroup is 4 wavefronts: S of them split the K loop of one tile (word w of
+//     the reference's K order (kh*KW + kw)*C_pack + ic goes to wavefront w % S of the tile), so
+//     it covers 4/S pixel tiles.  S = 1 for layers with many pixels (no exchange at all), 2 or 4
+//     where the tiles alone would leave most of the chip idle; the partial tiles then meet in
+//     LDS and each wavefront finishes 4/S of the tile's four blocks;
+//   * weights are the MFMA A side (rows = accumulator registers), pixels the B side (rows =
+//     lanes), so a store instruction writes 32 consecutive pixels of one NCHW plane;
+//   * an activation fragment is 32 pixels x 64 channels of one kernel tap: lane (pixel, half)
+//     loads its 16 bytes straight from P4 (k_quantize_f4's output) at the tap's input pixel,
+//     or takes the padding value: zeros for ternary inputs, +1 nibbles for binary ones (the
+//     reference's fill, src/tnns/ternarize2row_avx2.c:748-755, src/tnns/binarize2row_avx2.c:151);
+//   * the padding words that round K up to a multiple of 4 are skipped: their products are zero
+//     except for BNN, whose epilogue constant counts the real words only.
+struct ConvFrag {
+    v4i w[2], x[2];
+    bool in[2];   // x[b] holds a real input pixel (else the padding value replaces it)
+};
+
+template <bool ABIN, int S>
+__global__ __launch_bounds__(256) void k_conv_f4(const uint4* __restrict__ P4, const uint4* __restrict__ Wf,
+                                                 float* __restrict__ Y, int M, int KN, int OHW, int KB,
+                                                 int bias, int form, float alpha, FastDiv dOHW, ConvGeom cg) {
+    constexpr int NB = 3;                 // register sets of fragments: NB - 1 steps of loads in flight
+    constexpr int PUB = 4 - 4 / S;        // blocks a wavefront hands to the others of its tile
+    __shared__ float4 red[S > 1 ? 4 * PUB * 4 * 64 : 1];   // [wavefront][slot][e / 4][lane]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ks = wave % S, pt = wave / S;   // K share and pixel tile of this wavefront
+    const int h = lane >> 5, lr = lane & 31;
+    const int px0 = (blockIdx.x * (4 / S) + pt) * 64, kn0 = blockIdx.y * 64;
+
+    int ih0[2], iw0[2];
+    uint32_t pb[2];
+#pragma unroll
+    for (int b = 0; b < 2; b++) {
+        const uint32_t q = (uint32_t)min(px0 + 32 * b + lr, M - 1);
+        const uint32_t n = fastdiv(q, dOHW);
+        const uint32_t pix = q - n * (uint32_t)OHW;
+        const int oh = (int)fastdiv(pix, cg.dOW), ow = (int)pix - oh * cg.OW;
+        ih0[b] = oh * cg.H_stride - cg.H_pad;
+        iw0[b] = ow * cg.W_stride - cg.W_pad;
+        pb[b] = n * (uint32_t)(cg.CP * cg.H * cg.W);   // image n of P4[n][C_pack][pixel]
+    }
+    const int HWin = cg.H * cg.W;
+    const int rbmax = (KN + 31) / 32 - 1;
+    const uint4* wb[2];
+#pragma unroll
+    for (int a = 0; a < 2; a++) wb[a] = Wf + (size_t)min(kn0 / 32 + a, rbmax) * KB * 64 + lane;
+
+    v16f acc[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[a][b][e] = 0.0f;
+
+    const uint32_t fillv = ABIN ? 0x22222222u : 0u;
+    // All four loads of a step are unconditional (a tap outside the image reads pixel 0 of its
+    // image and is replaced by the padding value before use) and issued through inline asm, so
+    // that they leave when the code says so -- two steps ahead of the step being multiplied --
+    // and not where the compiler would sink them, next to their use.  The kernel counts them by
+    // hand: `arrive` waits until at most 8 loads (two steps) are outstanding and ties that wait to
+    // the registers of the step about to be used.
+    auto ld16 = [](v4i& dst, const uint4* src) {
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(dst) : "v"(src) : "memory");
+    };
+    auto load = [&](int w, ConvFrag& f) {   // w is wave-uniform
+        const int tap = (int)fastdiv((uint32_t)w, cg.dCP), ic = w - tap * cg.CP;
+        const int kh = (int)fastdiv((uint32_t)tap, cg.dKW), kw = tap - kh * cg.KW;
+#pragma unroll
+        for (int a = 0; a < 2; a++) ld16(f.w[a], wb[a] + (size_t)w * 64);
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            const int ih = ih0[b] + kh, iw = iw0[b] + kw;
+            const bool in = (unsigned)ih < (unsigned)cg.H && (unsigned)iw < (unsigned)cg.W;
+            const size_t o = (size_t)(pb[b] + (uint32_t)(ic * HWin + (in ? ih * cg.W + iw : 0))) * 2 + h;
+            ld16(f.x[b], P4 + o);
+            f.in[b] = in;
+        }
+    };
+    auto arrive = [](ConvFrag& f, auto outstanding) {
+        asm volatile("s_waitcnt vmcnt(%4)"
+                     : "+v"(f.w[0]), "+v"(f.w[1]), "+v"(f.x[0]), "+v"(f.x[1])
+                     : "n"(decltype(outstanding)::value)
+                     : "memory");
+    };
+    auto compute = [&](const ConvFrag& f) {
+        v8i x[2], wv[2];
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) x[b][i] = f.in[b] ? f.x[b][i] : (int)fillv;
+#pragma unroll
+            for (int i = 4; i < 8; i++) x[b][i] = 0;
+        }
+#pragma unroll
+        for (int a = 0; a < 2; a++) wv[a] = v8i{f.w[a][0], f.w[a][1], f.w[a][2], f.w[a][3], 0, 0, 0, 0};
+        // cbsz = blgp = 4: both operands E2M1, unscaled (see mfma<true>)
+#pragma unroll
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+            for (int b = 0; b < 2; b++)
+                acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wv[a], x[b], acc[a][b], 4, 4, 0, 0, 0, 0);
+    };
+
+    // The register sets rotate by name (the loop is unrolled by NB); loads past the last word
+    // re-read it and are not multiplied (whole rounds of NB steps).
+    const int K = cg.K;
+    ConvFrag f[NB];
+    std::integral_constant<int, 4 * (NB - 1)> ahead;
+    int w = ks;
+#pragma unroll
+    for (int j = 0; j < NB - 1; j++) load(min(w + S * j, K - 1), f[j]);
+    for (; w < K; w += S * NB) {
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+            load(min(w + S * (j + NB - 1), K - 1), f[(j + NB - 1) % NB]);
+            arrive(f[j], ahead);
+            if (j == 0 || w + S * j < K) compute(f[j]);
+        }
+    }
+    // the loads still in flight target live registers: drain them before anything reuses those
+#pragma unroll
+    for (int j = 0; j < NB; j++) arrive(f[j], std::integral_constant<int, 0>{});
+
+    // Block id = 2*a + b; wavefront ks of a tile finishes the blocks with id % S == ks and hands
+    // the others over through LDS.  Every copy below names its accumulator registers statically,
+    // under a wave-uniform branch, so that no register array is indexed at run time.
+    auto for_blocks = [&](auto&& fn) {
+        fn(std::integral_constant<int, 0>{});
+        fn(std::integral_constant<int, 1>{});
+        fn(std::integral_constant<int, 2>{});
+        fn(std::integral_constant<int, 3>{});
+    };
+    if constexpr (S > 1) {
+        for_blocks([&](auto blk_tag) {
+            constexpr int BLK = decltype(blk_tag)::value;
+            if (BLK % S != ks) {
+                // slot of BLK among the blocks wavefront ks does not own
+                const int slot = S == 4 ? (BLK < ks ? BLK : BLK - 1) : BLK / 2;
+                float4* dst = red + (size_t)((wave * PUB + slot) * 4) * 64 + lane;
+                const v16f& c = acc[BLK >> 1][BLK & 1];
+#pragma unroll
+                for (int e4 = 0; e4 < 4; e4++)
+                    dst[e4 * 64] = make_float4(c[4 * e4], c[4 * e4 + 1], c[4 * e4 + 2], c[4 * e4 + 3]);
+            }
+        });
+        __syncthreads();
+    }
+    const bool le_form = form == 0;
+    for_blocks([&](auto blk_tag) {
+        constexpr int BLK = decltype(blk_tag)::value;
+        if (BLK % S == ks) {
+            v16f mine = acc[BLK >> 1][BLK & 1];
+            if constexpr (S > 1) {
+#pragma unroll
+                for (int v = 0; v < S; v++) {
+                    if (v != BLK % S) {   // source wavefront pt*S + v holds BLK in the slot computed as above
+                        const int slot = S == 4 ? (BLK < v ? BLK : BLK - 1) : BLK / 2;
+                        const float4* src = red + (size_t)(((pt * S + v) * PUB + slot) * 4) * 64 + lane;
+#pragma unroll
+                        for (int e4 = 0; e4 < 4; e4++) {
+                            const float4 t = src[e4 * 64];
+                            mine[4 * e4] += t.x;
+                            mine[4 * e4 + 1] += t.y;
+                            mine[4 * e4 + 2] += t.z;
+                            mine[4 * e4 + 3] += t.w;
+                        }
+                    }
+                }
+            }
+            // accumulator e: kernel = 32*a + 8*(e/4) + 4*(lane/32) + e%4, pixel = 32*b + lane%32
+            constexpr int a = BLK >> 1, b = BLK & 1;
+            const int q = px0 + 32 * b + lr;
+            const uint32_t qc = (uint32_t)min(q, M - 1);
+            const uint32_t img = fastdiv(qc, dOHW);
+            float* yq = Y + (size_t)img * KN * OHW + (qc - img * (uint32_t)OHW);
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int p = kn0 + 32 * a + 8 * (e >> 2) + 4 * h + (e & 3);
+                const int r = (int)mine[e] - bias;
+                const float fr = (float)r;
+                // form 0: scale when f <= 0 (a zero becomes 0 * alpha); form 1: scale when r < 0
+                const bool scale = le_form ? (fr <= 0.0f) : (r < 0);
+                const float fv = scale ? fr * alpha : fr;
+                if (q < M && p < KN) yq[(size_t)p * OHW] = fv;
+            }
+        }
+    });
+}
+
 template <bool F4, bool SWAP>
 hipError_t launch_gemm(const uint4* Pf, const uint4* Qf, float* Y, int M, int KN, int OHW, int KB,
                        int bias, int form, float alpha, hipStream_t st) {
@@ -326,6 +523,41 @@ hipError_t launch_mfma_gemm(bool f4, int type, const void* d_af, const void* d_b
     }
     return swap ? launch_gemm<false, true>(Bf, Af, d_y, (int)M, KN, OHW, KB, bias, form, alpha, st)
                 : launch_gemm<false, false>(Af, Bf, d_y, (int)M, KN, OHW, KB, bias, form, alpha, st);
+}
+
+hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const ConvGeom& cg, int N, int KN,
+                          int K_unpack, float alpha, float* d_y, hipStream_t st) {
+    const int OHW = cg.OH * cg.OW;
+    const int64_t M = (int64_t)N * OHW;
+    const int KB = round4(cg.K);
+    // BNN: the channel lanes past C are +1 in both operands (see launch_mfma_gemm); padding words are skipped
+    const int bias = type == kBNN ? 64 * cg.K - K_unpack : 0;
+    const int form = type == kTNN ? 0 : 1;
+    // K split: enough wavefronts to occupy the chip's 1024 SIMDs, but no exchange where the tiles
+    // alone do that (a tile = 64 kernels x 64 pixels)
+    const int64_t tiles = ((M + 63) / 64) * ((KN + 63) / 64);
+    int split = tiles >= 1024 ? 1 : (tiles >= 512 ? 2 : 4);
+    static const char* tune = getenv("FTNN_CONV_SPLIT");   // tuning aid: force the K split
+    if (tune) split = atoi(tune);
+    dim3 grid((unsigned)(((M + 63) / 64 + 4 / split - 1) / (4 / split)), (unsigned)((KN + 63) / 64));
+    if (M > 0x7fffff00LL || grid.y > 65535) return hipErrorInvalidValue;   // pixel indices stay below 2^31
+    const uint4* P4 = static_cast<const uint4*>(d_p4);
+    const uint4* Wf = static_cast<const uint4*>(d_wf);
+    const FastDiv dOHW = make_fastdiv((uint32_t)OHW);
+    const bool abin = type == kBTN || type == kBNN;
+#define FTNN_CONV(S_)                                                                                            \
+    if (split == S_) {                                                                                           \
+        if (abin)                                                                                                \
+            hipLaunchKernelGGL((k_conv_f4<true, S_>), grid, dim3(256), 0, st, P4, Wf, d_y, (int)M, KN, OHW, KB,  \
+                               bias, form, alpha, dOHW, cg);                                                     \
+        else                                                                                                     \
+            hipLaunchKernelGGL((k_conv_f4<false, S_>), grid, dim3(256), 0, st, P4, Wf, d_y, (int)M, KN, OHW, KB, \
+                               bias, form, alpha, dOHW, cg);                                                     \
+        return hipGetLastError();                                                                                \
+    }
+    FTNN_CONV(1) FTNN_CONV(2) FTNN_CONV(4)
+#undef FTNN_CONV
+    return hipErrorInvalidValue;
 }
 
 hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* d_b, int64_t M, int OHW,

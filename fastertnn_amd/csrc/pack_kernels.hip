@@ -76,6 +76,53 @@ __global__ __launch_bounds__(256) void k_quantize_pixels(const float* __restrict
     }
 }
 
+// Quantise straight into the operand form of the fp4 matrix-core layer kernel: one E2M1 nibble
+// per channel (0x2 = +1, 0x0 = 0, 0xA = -1; low nibble = even channel), 32 bytes per pixel and
+// 64 channels, in planes of 64 channels: P4[n][C_pack][pixel][32 bytes], so that the 32
+// consecutive pixels of a matrix-core fragment are (for stride 1) one contiguous KiB.  Channels past C read as the reference's padding
+// lanes: zero for ternary inputs (src/tnns/ternarize2row_avx2.c:440-441), +1 for binary ones
+// (cleared bits, src/tnns/binarize2row_avx2.c:151).  Same block shape and loads as
+// k_quantize_pixels; a thread's 8 channels are one dword, transposed through LDS so that a
+// pixel's 32 bytes leave contiguously.
+template <bool TERN>
+__global__ __launch_bounds__(256) void k_quantize_f4(const float* __restrict__ x,
+                                                     const float* __restrict__ thr, int C, int HW,
+                                                     int CP, uint32_t* __restrict__ P4) {
+    __shared__ uint32_t s_dw[32 * 9];
+    const int px = threadIdx.x & 31, oct = threadIdx.x >> 5;
+    const int p = blockIdx.x * 32 + px;
+    const int ic = blockIdx.y, n = blockIdx.z;
+    const float t = thr[n];
+    const int c0 = ic * 64 + oct * 8;
+    uint32_t dw = TERN ? 0u : 0x22222222u;
+    if (p < HW) {
+        const float* xp = x + ((size_t)n * C + c0) * HW + p;
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = (c0 + j < C) ? xp[(size_t)j * HW] : 0.0f;
+        dw = 0u;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            uint32_t nib;
+            if (TERN) {
+                // strict compares, src/tnns/ternarize2row_avx2.c:443-449
+                nib = v[j] < -t ? 0xAu : (v[j] > t ? 0x2u : 0x0u);
+                if (c0 + j >= C) nib = 0x0u;
+            } else {
+                // src/tnns/binarize2row_avx2.c:19-21
+                nib = v[j] < t ? 0xAu : 0x2u;
+                if (c0 + j >= C) nib = 0x2u;
+            }
+            dw |= nib << (4 * j);
+        }
+    }
+    s_dw[px * 9 + oct] = dw;
+    __syncthreads();
+    const int wp = threadIdx.x >> 3, wo = threadIdx.x & 7;
+    const int q = blockIdx.x * 32 + wp;
+    if (q < HW) P4[(((size_t)n * CP + ic) * HW + q) * 8 + wo] = s_dw[wp * 9 + wo];
+}
+
 // One wavefront ballot per 64-bit word: rows of J consecutive floats.
 // MODE 0: ternary thresholds, 1: binary threshold, 2: exact values {-1,0,+1}
 // (bitpacking2).  P2ROW: write straight into Packing-2 rows of 2*J/64 words
@@ -361,6 +408,16 @@ hipError_t launch_quantize(bool ternary, const float* d_x, const float* d_thr, i
             hipLaunchKernelGGL((k_quantize_pixels<false>), grid, dim3(256), 0, st, d_x, d_thr, C,
                                HW, CP, P);
     }
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_f4(bool ternary, const float* d_x, const float* d_thr, int N, int C, int H, int W,
+                              void* d_p4, hipStream_t st) {
+    const int CP = cpack_of(C), HW = H * W;
+    dim3 grid((HW + 31) / 32, CP, N);
+    uint32_t* P4 = static_cast<uint32_t*>(d_p4);
+    if (ternary) hipLaunchKernelGGL((k_quantize_f4<true>), grid, dim3(256), 0, st, d_x, d_thr, C, HW, CP, P4);
+    else hipLaunchKernelGGL((k_quantize_f4<false>), grid, dim3(256), 0, st, d_x, d_thr, C, HW, CP, P4);
     return hipGetLastError();
 }
 

@@ -206,6 +206,21 @@ FTNN_API int ftnn_conv(int type, const float *d_x, const float *d_thr, const int
               int W_stride, float prelu_alpha, void *d_scratch, float *d_y, void *stream);
 
 /*
+ * The same layer on an explicit engine (no counterpart in the reference; same bits on either):
+ * FTNN_ENGINE_VALU      quantise to bit planes, vector-ALU popcount GEMM with implicit im2row;
+ * FTNN_ENGINE_MFMA_F4   quantise to fp4 nibbles, expand the weights into matrix-core fragments
+ *                       (in d_scratch) and run the fp4 matrix-core layer kernel;
+ * FTNN_ENGINE_AUTO      what ftnn_conv does: ftnn_select_conv_engine()'s choice.
+ * ftnn_conv_scratch_bytes() covers every engine.
+ */
+FTNN_API int ftnn_select_conv_engine(int type, int N, int C, int H, int W, int KN, int KH, int KW, int H_pad,
+                                     int W_pad, int H_stride, int W_stride);
+FTNN_API int ftnn_conv_engine(int engine, int type, const float *d_x, const float *d_thr, const int64_t *d_qw,
+                              int N, int C, int H, int W, int KN, int KH, int KW, int H_pad, int W_pad,
+                              int H_stride, int W_stride, float prelu_alpha, void *d_scratch, float *d_y,
+                              void *stream);
+
+/*
  * A chain of conv layers with device-resident activations: the e2e mode of the reference's
  * layer driver (src/timing_layers.c:182-207 feeds each layer's output to the next one), here
  * without the host round trip per layer.  All device memory (two activation buffers, the

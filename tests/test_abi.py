@@ -98,10 +98,17 @@ def test_engine_selection_and_scratch_sizes_need_no_device():
     assert lib.mm_scratch_bytes(lib.ENGINE_AUTO, 0, 8192, 1, 1, 8192, 512) == 2 * 256 * 512 * 1024
     assert lib._L.ftnn_expand_bytes(lib.ENGINE_MFMA_F4, 100, 6) == 4 * 8 * 1024
     assert lib._L.ftnn_expand_bytes(lib.ENGINE_VALU, 100, 6) == 0
-    # conv scratch: the quantised input, plus dense rows and weights when C <= 32 packs several taps per word
-    assert lib.conv_scratch_bytes(0, 2, 64, 8, 8, 16, 3, 3, 1, 1) == lib.pack_scratch_bytes(2, 64, 8, 8, 1)
-    dense = lib.conv_scratch_bytes(0, 2, 3, 32, 32, 16, 7, 7, 3, 2)
-    assert dense == 2 * 32 * 32 * 16 + 2 * 16 * 16 * 4 * 16 + 16 * 4 * 16
+    # conv scratch covers either layer engine.  Vector ALU: the quantised input (16 bytes per pixel and 64
+    # channels), plus dense rows and weights when C <= 32 packs several taps per word.  fp4 matrix cores: 32 bytes
+    # per pixel and 64 channels, plus 1 KiB per 32 kernels and word of the rounded-up row.
+    assert lib.pack_scratch_bytes(2, 64, 8, 8, 1) == 2 * 8 * 8 * 16
+    assert lib.conv_scratch_bytes(0, 2, 64, 8, 8, 16, 3, 3, 1, 1) == 2 * 8 * 8 * 32 + 1 * 12 * 1024
+    valu_dense = 2 * 32 * 32 * 16 + 2 * 16 * 16 * 4 * 16 + 16 * 4 * 16
+    fp4 = 2 * 32 * 32 * 32 + 1 * 52 * 1024
+    assert lib.conv_scratch_bytes(0, 2, 3, 32, 32, 16, 7, 7, 3, 2) == max(valu_dense, fp4)
+    # layer engine: fp4 wherever the dense re-packing does not apply and fp32 accumulation stays exact
+    assert lib.select_conv_engine(0, 1, 256, 56, 56, 256, 3, 3, 1, 1) == lib.ENGINE_MFMA_F4
+    assert lib.select_conv_engine(0, 32, 3, 224, 224, 64, 7, 7, 3, 2) == lib.ENGINE_VALU
 
 
 def test_missing_library_is_an_import_error(tmp_path):

@@ -49,3 +49,7 @@ def test_layer_device_api(hip, oracle, typ, si, batch):
     _same_bits(y_d.cpu().numpy(), y_o, "GEMM output")
     yc_d = hip.conv(typ, x_d, thr_d, qw_d, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], L["alpha"])
     _same_bits(yc_d.cpu().numpy(), y_o, "conv output")
+    for eng in (hip.ENGINE_VALU, hip.ENGINE_MFMA_F4):   # the layer on each engine explicitly
+        ye_d = hip.conv(typ, x_d, thr_d, qw_d, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], L["alpha"],
+                        engine=eng)
+        _same_bits(ye_d.cpu().numpy(), y_o, "conv output, engine %d" % eng)

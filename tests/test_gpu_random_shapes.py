@@ -42,6 +42,10 @@ def test_random_layers(hip, oracle, chunk):
         x_d, thr_d, qw_d = (torch.from_numpy(np.ascontiguousarray(v)).cuda() for v in (L["x"], L["thr"], qw))
         got = hip.conv(typ, x_d, thr_d, qw_d, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], L["alpha"])
         assert got.cpu().numpy().tobytes() == want.tobytes(), "fused layer"
+        for eng in (hip.ENGINE_VALU, hip.ENGINE_MFMA_F4):
+            got = hip.conv(typ, x_d, thr_d, qw_d, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], L["alpha"],
+                           engine=eng)
+            assert got.cpu().numpy().tobytes() == want.tobytes(), "fused layer, engine %d" % eng
         rows = hip.quantize_im2row(x_d, thr_d, L["kh"], L["kw"], L["pad"], L["stride"], at)
         oh, ow = want.shape[2], want.shape[3]
         kk, ku = ((L["c"] + 63) // 64) * L["kh"] * L["kw"], L["c"] * L["kh"] * L["kw"]
