@@ -162,18 +162,100 @@ static float* host_mm(int type, int64_t* a, int64_t* b, int N, int OH, int OW, i
     return y;
 }
 
+// bytes of the two regions of the matrix-core layer path: P4 (32 bytes per pixel and 64 channels),
+// then the fp4 fragments of the weights
+int64_t conv_f4_p4_bytes(int N, int C, int H, int W) {
+    return ((int64_t)N * H * W * cpack_of(C) * 32 + 255) / 256 * 256;
+}
+
+// the same region for a few-channel layer on the dense fp4 path: nibble pixels, then the dense rows
+int64_t conv_f4_dense_bytes(int N, int C, int H, int W, int KH, int KW, int OH, int OW) {
+    int T, Kd;
+    dense_applies(C, KH, KW, &T, &Kd);
+    return dense_f4_pq_bytes(N, H, W) + ((int64_t)N * OH * OW * Kd * 32 + 255) / 256 * 256;
+}
+
+// operand region of the fp4 layer for this shape, whichever of the two forms it takes
+int64_t conv_f4_operand_bytes(int N, int C, int H, int W, int KH, int KW, int OH, int OW) {
+    return dense_f4_applies(C, KH, KW) ? conv_f4_dense_bytes(N, C, H, W, KH, KW, OH, OW) : conv_f4_p4_bytes(N, C, H, W);
+}
+
+// words per expanded weight row on the fp4 layer path
+int conv_f4_weight_words(int C, int KH, int KW) {
+    int T, Kd;
+    if (dense_f4_applies(C, KH, KW)) {
+        dense_applies(C, KH, KW, &T, &Kd);
+        return round4(Kd);
+    }
+    return round4(cpack_of(C) * KH * KW);
+}
+
 // the matrix-core layer with the weights already expanded (d_wf); d_p4 takes the quantised input
 int conv_f4_expanded(int type, const float* d_x, const float* d_thr, const void* d_wf, int N, int C, int H,
                            int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride, int W_stride,
-                           float prelu_alpha, void* d_p4, float* d_y, hipStream_t st) {
+                           float prelu_alpha, void* d_p4, float* d_y, hipStream_t st, const QuantOut& qo) {
     const int OH = out_dim(H, H_pad, KH, H_stride), OW = out_dim(W, W_pad, KW, W_stride);
     const bool act_ternary = (type == kTNN || type == kTBN);
-    hipError_t e = launch_quantize_f4(act_ternary, d_x, d_thr, N, C, H, W, d_p4, st);
+    hipError_t e = hipSuccess;
+    if (dense_f4_applies(C, KH, KW)) {
+        // few channels: several taps per 64-lane word, materialised per output pixel; the layer is then a 1x1
+        // layer with Kd words per pixel over the OH x OW output pixels
+        if (!d_x) return fail(FTNN_EINVAL, "a few-channel layer takes fp32 input");
+        int T, Kd;
+        dense_applies(C, KH, KW, &T, &Kd);
+        void* d_a4 = static_cast<char*>(d_p4) + dense_f4_pq_bytes(N, H, W);
+        e = launch_dense_rows_f4(act_ternary, d_x, d_thr, N, C, H, W, H_pad, W_pad, KH, KW, H_stride, W_stride, d_p4,
+                                 d_a4, st);
+        if (e != hipSuccess) return hip_fail(e, "fp4 dense rows launch");
+        const ConvGeom cg = {OH, OW, Kd, OH, OW, 1, Kd, 0, 0, 1, 1,
+                             make_fastdiv((uint32_t)OW), make_fastdiv((uint32_t)Kd), make_fastdiv(1u)};
+        e = launch_conv_f4(type, d_a4, d_wf, cg, N, KN, C * KH * KW, prelu_alpha, d_y, st, qo);
+        return e == hipSuccess ? FTNN_OK : hip_fail(e, "fp4 conv launch");
+    }
+    if (d_x) e = launch_quantize_f4(act_ternary, d_x, d_thr, N, C, H, W, d_p4, st);   // else d_p4 is ready
     if (e != hipSuccess) return hip_fail(e, "fp4 quantize launch");
     const ConvGeom cg = {H, W, cpack_of(C), OH, OW, KW, cpack_of(C) * KH * KW, H_pad, W_pad, H_stride, W_stride,
                          make_fastdiv((uint32_t)OW), make_fastdiv((uint32_t)cpack_of(C)), make_fastdiv((uint32_t)KW)};
-    e = launch_conv_f4(type, d_p4, d_wf, cg, N, KN, C * KH * KW, prelu_alpha, d_y, st);
+    e = launch_conv_f4(type, d_p4, d_wf, cg, N, KN, C * KH * KW, prelu_alpha, d_y, st, qo);
     return e == hipSuccess ? FTNN_OK : hip_fail(e, "fp4 conv launch");
+}
+
+// the vector-ALU layer: quantise to bit planes, then the implicit-im2row GEMM (or, for few channels, the dense
+// re-packing and the plain GEMM)
+int conv_valu(int type, const float* d_x, const float* d_thr, const int64_t* d_qw, int N, int C, int H, int W,
+              int KN, int KH, int KW, int H_pad, int W_pad, int H_stride, int W_stride, float prelu_alpha,
+              void* d_scratch, float* d_y, hipStream_t st, const QuantOut& qo, bool weights_prepared) {
+    const int OH = out_dim(H, H_pad, KH, H_stride), OW = out_dim(W, W_pad, KW, W_stride);
+    const bool act_ternary = (type == kTNN || type == kTBN);
+    const bool w_ternary = (type == kTNN || type == kBTN);
+    hipError_t e = launch_quantize(act_ternary, d_x, d_thr, N, C, H, W, d_scratch, st);
+    if (e != hipSuccess) return hip_fail(e, "quantize launch");
+    int T, Kd;
+    if (dense_applies(C, KH, KW, &T, &Kd)) {
+        // few channels: re-pack both operands with several taps per word and run the plain GEMM
+        char* base = static_cast<char*>(d_scratch);
+        const int64_t p_bytes = (ftnn_pack_scratch_bytes(N, C, H, W, act_ternary) + 255) / 256 * 256;
+        const int64_t rows_bytes =
+            ((int64_t)N * OH * OW * round4(Kd) * (act_ternary ? 16 : 8) + 255) / 256 * 256;
+        int64_t* d_rows = reinterpret_cast<int64_t*>(base + p_bytes);
+        const int64_t* d_wd = d_qw;   // prepared weights are the re-packed rows already
+        e = launch_dense_rows(act_ternary, d_scratch, N, C, H, W, H_pad, W_pad, KH, KW, H_stride, W_stride,
+                              d_rows, st);
+        if (e != hipSuccess) return hip_fail(e, "dense rows launch");
+        if (!weights_prepared) {
+            int64_t* d_tmp = reinterpret_cast<int64_t*>(base + p_bytes + rows_bytes);
+            e = launch_dense_weights(w_ternary, d_qw, KN, C, KH, KW, d_tmp, st);
+            if (e != hipSuccess) return hip_fail(e, "dense weights launch");
+            d_wd = d_tmp;
+        }
+        e = launch_mm(type, d_rows, d_wd, (int64_t)N * OH * OW, OH * OW, KN, round4(Kd), C * KH * KW,
+                      prelu_alpha, d_y, st, qo);
+        return e == hipSuccess ? FTNN_OK : hip_fail(e, "mm launch");
+    }
+    const ConvGeom cg = {H, W, cpack_of(C), OH, OW, KW, cpack_of(C) * KH * KW, H_pad, W_pad, H_stride, W_stride,
+                         make_fastdiv((uint32_t)OW), make_fastdiv((uint32_t)cpack_of(C)), make_fastdiv((uint32_t)KW)};
+    e = launch_mm_implicit(type, d_scratch, d_qw, cg, N, KN, C * KH * KW, prelu_alpha, d_y, st, qo);
+    return e == hipSuccess ? FTNN_OK : hip_fail(e, "implicit-im2row mm launch");
 }
 
 }  // namespace ftnn
@@ -197,18 +279,13 @@ int64_t ftnn_pack_scratch_bytes(int N, int C, int H, int W, int ternary) {
     return (int64_t)N * H * W * cpack_of(C) * (ternary ? 16 : 8);
 }
 
-// bytes of the two regions of the matrix-core layer path: P4 (32 bytes per pixel and 64 channels),
-// then the fp4 fragments of the weights
-static int64_t conv_f4_p4_bytes(int N, int C, int H, int W) {
-    return ((int64_t)N * H * W * cpack_of(C) * 32 + 255) / 256 * 256;
-}
-
 // Layer engine by shape, from measurements on MI355X: the fp4 matrix-core kernel wins wherever it
-// applies except on the few-channel layers that the dense re-packing shrinks.
+// applies.
 static int select_conv_engine(int type, int N, int C, int H, int W, int KN, int KH, int KW, int OH, int OW) {
     (void)type; (void)N; (void)H; (void)W; (void)KN; (void)OH; (void)OW;
     int T, Kd;
-    if (dense_applies(C, KH, KW, &T, &Kd)) return FTNN_ENGINE_VALU;
+    // few channels: the dense re-packing feeds the matrix cores for C <= 8, the vector ALU beyond
+    if (dense_applies(C, KH, KW, &T, &Kd)) return C <= 8 ? FTNN_ENGINE_MFMA_F4 : FTNN_ENGINE_VALU;
     if (64LL * cpack_of(C) * KH * KW >= (1LL << 24)) return FTNN_ENGINE_VALU;   // fp32 accumulation must stay exact
     return FTNN_ENGINE_MFMA_F4;
 }
@@ -235,7 +312,10 @@ int64_t ftnn_conv_scratch_bytes(int type, int N, int C, int H, int W, int KN, in
         bytes += (int64_t)KN * round4(Kd) * (wt ? 16 : 8);
     }
     // enough for either engine, so that one buffer serves ftnn_conv and ftnn_conv_engine
-    const int64_t f4 = conv_f4_p4_bytes(N, C, H, W) + mfma_fragment_bytes(true, KN, round4(cpack_of(C) * KH * KW));
+    // fp4: operand region, fragments of the weights and, on the dense path, the re-packed weight rows
+    int64_t f4 = conv_f4_operand_bytes(N, C, H, W, KH, KW, OH, OW) +
+                 (mfma_fragment_bytes(true, KN, conv_f4_weight_words(C, KH, KW)) + 255) / 256 * 256;
+    if (dense_f4_applies(C, KH, KW)) f4 += (int64_t)KN * conv_f4_weight_words(C, KH, KW) * (wt ? 16 : 8);
     return bytes > f4 ? bytes : f4;
 }
 
@@ -384,45 +464,107 @@ int ftnn_conv_engine(int engine, int type, const float* d_x, const float* d_thr,
         return fail(FTNN_EINVAL, "d_scratch and d_qw must be 16-byte aligned");
     if ((int64_t)N * OH * OW > 0x7fffffffLL) return fail(FTNN_EINVAL, "more than 2^31-1 output rows");
     if (engine == FTNN_ENGINE_AUTO) engine = select_conv_engine(type, N, C, H, W, KN, KH, KW, OH, OW);
-    const bool act_ternary = (type == kTNN || type == kTBN);
     const bool w_ternary = (type == kTNN || type == kBTN);
     if (engine == FTNN_ENGINE_MFMA_F4) {
-        const int Kw = round4(cpack_of(C) * KH * KW);
+        const int Kw = conv_f4_weight_words(C, KH, KW);
         if (64LL * Kw >= (1LL << 24))
             return fail(FTNN_EINVAL, "K too long for exact fp32 accumulation; use the vector-ALU engine");
-        if ((int64_t)N * H * W * cpack_of(C) > 0x7fffffffLL)
+        if ((int64_t)N * H * W * cpack_of(C) > 0x7fffffffLL || (int64_t)N * OH * OW * Kw > 0x7fffffffLL)
             return fail(FTNN_EINVAL, "more than 2^31-1 input pixel words");
-        void* d_wf = static_cast<char*>(d_scratch) + conv_f4_p4_bytes(N, C, H, W);
-        hipError_t e = launch_mfma_expand(true, w_ternary, d_qw, KN, Kw, d_wf, (hipStream_t)stream);
+        char* d_wf = static_cast<char*>(d_scratch) + conv_f4_operand_bytes(N, C, H, W, KH, KW, OH, OW);
+        const int64_t* rows = d_qw;
+        hipError_t e;
+        if (dense_f4_applies(C, KH, KW)) {   // the weights take the same re-packing first
+            int64_t* d_wd = reinterpret_cast<int64_t*>(d_wf + (mfma_fragment_bytes(true, KN, Kw) + 255) / 256 * 256);
+            e = launch_dense_weights(w_ternary, d_qw, KN, C, KH, KW, d_wd, (hipStream_t)stream);
+            if (e != hipSuccess) return hip_fail(e, "dense weights launch");
+            rows = d_wd;
+        }
+        e = launch_mfma_expand(true, w_ternary, rows, KN, Kw, d_wf, (hipStream_t)stream);
         if (e != hipSuccess) return hip_fail(e, "weight expansion launch");
         return conv_f4_expanded(type, d_x, d_thr, d_wf, N, C, H, W, KN, KH, KW, H_pad, W_pad, H_stride, W_stride,
-                                prelu_alpha, d_scratch, d_y, (hipStream_t)stream);
+                                prelu_alpha, d_scratch, d_y, (hipStream_t)stream, QuantOut());
     }
     if (engine != FTNN_ENGINE_VALU) return fail(FTNN_EINVAL, "layer engine %d (vector ALU and fp4 only)", engine);
-    hipError_t e = launch_quantize(act_ternary, d_x, d_thr, N, C, H, W, d_scratch, (hipStream_t)stream);
-    if (e != hipSuccess) return hip_fail(e, "quantize launch");
+    return conv_valu(type, d_x, d_thr, d_qw, N, C, H, W, KN, KH, KW, H_pad, W_pad, H_stride, W_stride, prelu_alpha,
+                     d_scratch, d_y, (hipStream_t)stream, QuantOut(), false);
+}
+
+// Weights in the form the layer's engine reads them, made once per layer instead of once per call.
+static int64_t prepared_bytes(int type, int C, int KN, int KH, int KW, int64_t* tmp_off) {
+    const bool wt = (type == kTNN || type == kBTN);
+    const int engine = select_conv_engine(type, 1, C, KH, KW, KN, KH, KW, 1, 1);
     int T, Kd;
-    if (dense_applies(C, KH, KW, &T, &Kd)) {
-        // few channels: re-pack both operands with several taps per word and run the plain GEMM
-        char* base = static_cast<char*>(d_scratch);
-        const int64_t p_bytes = (ftnn_pack_scratch_bytes(N, C, H, W, act_ternary) + 255) / 256 * 256;
-        const int64_t rows_bytes =
-            ((int64_t)N * OH * OW * round4(Kd) * (act_ternary ? 16 : 8) + 255) / 256 * 256;
-        int64_t* d_rows = reinterpret_cast<int64_t*>(base + p_bytes);
-        int64_t* d_wd = reinterpret_cast<int64_t*>(base + p_bytes + rows_bytes);
-        e = launch_dense_rows(act_ternary, d_scratch, N, C, H, W, H_pad, W_pad, KH, KW, H_stride, W_stride,
-                              d_rows, (hipStream_t)stream);
-        if (e != hipSuccess) return hip_fail(e, "dense rows launch");
-        e = launch_dense_weights(w_ternary, d_qw, KN, C, KH, KW, d_wd, (hipStream_t)stream);
-        if (e != hipSuccess) return hip_fail(e, "dense weights launch");
-        e = launch_mm(type, d_rows, d_wd, (int64_t)N * OH * OW, OH * OW, KN, round4(Kd), C * KH * KW,
-                      prelu_alpha, d_y, (hipStream_t)stream);
-        return e == hipSuccess ? FTNN_OK : hip_fail(e, "mm launch");
+    const bool dense = dense_applies(C, KH, KW, &T, &Kd);
+    if (tmp_off) *tmp_off = 0;
+    if (engine == FTNN_ENGINE_MFMA_F4) {
+        const int64_t frag = (mfma_fragment_bytes(true, KN, conv_f4_weight_words(C, KH, KW)) + 255) / 256 * 256;
+        if (tmp_off) *tmp_off = frag;
+        // the dense path expands the re-packed rows, which need a place of their own
+        return frag + (dense_f4_applies(C, KH, KW) ? (int64_t)KN * round4(Kd) * (wt ? 16 : 8) : 0);
     }
-    const ConvGeom cg = {H, W, cpack_of(C), OH, OW, KW, cpack_of(C) * KH * KW, H_pad, W_pad, H_stride, W_stride,
-                         make_fastdiv((uint32_t)OW), make_fastdiv((uint32_t)cpack_of(C)), make_fastdiv((uint32_t)KW)};
-    e = launch_mm_implicit(type, d_scratch, d_qw, cg, N, KN, C * KH * KW, prelu_alpha, d_y, (hipStream_t)stream);
-    return e == hipSuccess ? FTNN_OK : hip_fail(e, "implicit-im2row mm launch");
+    return (int64_t)KN * (dense ? round4(Kd) : round4(cpack_of(C) * KH * KW)) * (wt ? 16 : 8);
+}
+
+int64_t ftnn_conv_weights_bytes(int type, int C, int KN, int KH, int KW) {
+    if (type < kTNN || type > kBNN || C <= 0 || KN <= 0 || KH <= 0 || KW <= 0) return 0;
+    return prepared_bytes(type, C, KN, KH, KW, nullptr);
+}
+
+int ftnn_conv_prepare_weights(int type, const int64_t* d_qw, int C, int KN, int KH, int KW, void* d_prepared,
+                              void* stream) {
+    if (type < kTNN || type > kBNN) return fail(FTNN_EINVAL, "unknown network type %d", type);
+    if (C <= 0 || KN <= 0 || KH <= 0 || KW <= 0) return fail(FTNN_EINVAL, "non-positive dimension");
+    if (!d_qw || !d_prepared || !aligned16(d_qw) || !aligned16(d_prepared))
+        return fail(FTNN_EINVAL, "null or misaligned device pointer");
+    const bool wt = (type == kTNN || type == kBTN);
+    hipStream_t st = (hipStream_t)stream;
+    int64_t tmp_off;
+    const int64_t bytes = prepared_bytes(type, C, KN, KH, KW, &tmp_off);
+    const int engine = select_conv_engine(type, 1, C, KH, KW, KN, KH, KW, 1, 1);
+    int T, Kd;
+    const bool dense = dense_applies(C, KH, KW, &T, &Kd);
+    hipError_t e;
+    if (engine == FTNN_ENGINE_MFMA_F4) {
+        const int64_t* rows = d_qw;
+        if (dense_f4_applies(C, KH, KW)) {
+            int64_t* d_wd = reinterpret_cast<int64_t*>(static_cast<char*>(d_prepared) + tmp_off);
+            e = launch_dense_weights(wt, d_qw, KN, C, KH, KW, d_wd, st);
+            if (e != hipSuccess) return hip_fail(e, "dense weights launch");
+            rows = d_wd;
+        }
+        e = launch_mfma_expand(true, wt, rows, KN, conv_f4_weight_words(C, KH, KW), d_prepared, st);
+        return e == hipSuccess ? FTNN_OK : hip_fail(e, "weight expansion launch");
+    }
+    if (dense) {
+        e = launch_dense_weights(wt, d_qw, KN, C, KH, KW, static_cast<int64_t*>(d_prepared), st);
+        return e == hipSuccess ? FTNN_OK : hip_fail(e, "dense weights launch");
+    }
+    e = hipMemcpyAsync(d_prepared, d_qw, (size_t)bytes, hipMemcpyDeviceToDevice, st);
+    return e == hipSuccess ? FTNN_OK : hip_fail(e, "weight copy");
+}
+
+int ftnn_conv_prepared(int type, const float* d_x, const float* d_thr, const void* d_prepared, int N, int C, int H,
+                       int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride, int W_stride,
+                       float prelu_alpha, void* d_scratch, float* d_y, void* stream) {
+    if (type < kTNN || type > kBNN) return fail(FTNN_EINVAL, "unknown network type %d", type);
+    int OH, OW;
+    int rc = check_conv_shape(N, C, H, W, H_pad, W_pad, KH, KW, H_stride, W_stride, &OH, &OW);
+    if (rc != FTNN_OK) return rc;
+    if (KN <= 0) return fail(FTNN_EINVAL, "non-positive kernel count");
+    if (!d_x || !d_thr || !d_prepared || !d_scratch || !d_y) return fail(FTNN_EINVAL, "null device pointer");
+    if (!aligned16(d_scratch) || !aligned16(d_prepared))
+        return fail(FTNN_EINVAL, "d_scratch and d_prepared must be 16-byte aligned");
+    if ((int64_t)N * OH * OW > 0x7fffffffLL) return fail(FTNN_EINVAL, "more than 2^31-1 output rows");
+    if (select_conv_engine(type, N, C, H, W, KN, KH, KW, OH, OW) == FTNN_ENGINE_MFMA_F4) {
+        if ((int64_t)N * H * W * cpack_of(C) > 0x7fffffffLL ||
+            (int64_t)N * OH * OW * conv_f4_weight_words(C, KH, KW) > 0x7fffffffLL)
+            return fail(FTNN_EINVAL, "more than 2^31-1 input pixel words");
+        return conv_f4_expanded(type, d_x, d_thr, d_prepared, N, C, H, W, KN, KH, KW, H_pad, W_pad, H_stride,
+                                W_stride, prelu_alpha, d_scratch, d_y, (hipStream_t)stream, QuantOut());
+    }
+    return conv_valu(type, d_x, d_thr, static_cast<const int64_t*>(d_prepared), N, C, H, W, KN, KH, KW, H_pad, W_pad,
+                     H_stride, W_stride, prelu_alpha, d_scratch, d_y, (hipStream_t)stream, QuantOut(), true);
 }
 
 int ftnn_conv(int type, const float* d_x, const float* d_thr, const int64_t* d_qw, int N, int C,

@@ -36,6 +36,23 @@ struct ConvGeom {
     FastDiv dOW, dCP, dKW;
 };
 
+// Fused hand-over to a following fp4 layer: instead of the fp32 result, a GEMM kernel writes the
+// next layer's quantised input, P4[n][ceil(KN/64)][pixel][32 bytes] (see launch_quantize_f4), from
+// the same fp32 values: mode 1 = ternary with thr[n] (strict compares), 2 = binary, 0 = off.
+// Kernels past KN in the last 64-channel word get the padding nibble.
+struct QuantOut {
+    void* p4 = nullptr;
+    const float* thr = nullptr;   // one threshold per batch item of the next layer
+    int mode = 0;
+};
+
+// the E2M1 nibble of one value under QuantOut mode 1 / 2 (src/tnns/ternarize2row_avx2.c:443-449,
+// src/tnns/binarize2row_avx2.c:19-21); `live` = false gives the padding lane of that mode
+__device__ __forceinline__ uint32_t quant_nibble(float v, float t, bool ternary, bool live) {
+    if (ternary) return live ? (v < -t ? 0xAu : (v > t ? 0x2u : 0x0u)) : 0x0u;
+    return live ? (v < t ? 0xAu : 0x2u) : 0x2u;
+}
+
 // record a failure text for ftnn_last_error(); returns `code`
 int fail(int code, const char* fmt, ...);
 
@@ -50,11 +67,12 @@ hipError_t launch_pack_gemm_operand(const float* d_x, int I, int J, int64_t* d_o
 // ---- mm_kernels.hip ----
 hipError_t launch_mm(int type, const int64_t* d_a, const int64_t* d_b, int64_t M, int OHW, int KN,
                      int Kw /* words per plane, multiple of 4 */, int K_unpack, float alpha,
-                     float* d_y, hipStream_t st);
+                     float* d_y, hipStream_t st, const QuantOut& qo = QuantOut());
 
 // GEMM straight from the channel-packed input P (no im2row matrix in memory)
 hipError_t launch_mm_implicit(int type, const void* d_p, const int64_t* d_b, const ConvGeom& cg, int N,
-                              int KN, int K_unpack, float alpha, float* d_y, hipStream_t st);
+                              int KN, int K_unpack, float alpha, float* d_y, hipStream_t st,
+                              const QuantOut& qo = QuantOut());
 // quantise only: fp32 NCHW -> P
 hipError_t launch_quantize(bool ternary, const float* d_x, const float* d_thr, int N, int C, int H, int W,
                            void* d_p, hipStream_t st);
@@ -70,6 +88,15 @@ hipError_t launch_dense_rows(bool ternary, const void* d_p, int N, int C, int H,
 hipError_t launch_dense_weights(bool ternary, const int64_t* d_qw, int KN, int C, int kH, int kW,
                                 int64_t* d_out, hipStream_t st);
 
+// the same for the fp4 layer kernel (C <= 8): quantise to one nibble dword per pixel (d_pq,
+// dense_f4_pq_bytes), then string T taps per 64-lane word into A4[n][Kd][output pixel][32 bytes] (d_a4), the
+// operand of launch_conv_f4 for a 1x1 layer with C_pack = Kd over the OH x OW output pixels
+bool dense_f4_applies(int C, int KH, int KW);
+int64_t dense_f4_pq_bytes(int N, int H, int W);
+hipError_t launch_dense_rows_f4(bool ternary, const float* d_x, const float* d_thr, int N, int C, int H, int W,
+                                int H_pad, int W_pad, int kH, int kW, int H_stride, int W_stride, void* d_pq,
+                                void* d_a4, hipStream_t st);
+
 // ---- mfma_kernels.hip: matrix-core formulation (int8 or fp4 operands expanded into d_scratch) ----
 int64_t mfma_fragment_bytes(bool f4, int64_t rows, int Kw);
 hipError_t launch_mfma_expand(bool f4, bool ternary, const int64_t* d_rows, int rows, int Kw, void* d_out,
@@ -83,14 +110,25 @@ hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* 
 // conv layer on the fp4 matrix cores: activations from launch_quantize_f4, weights as the fp4 fragments
 // launch_mfma_expand(true, ...) makes of the packed weight rows (Kw = round4(cg.K) words per row)
 hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const ConvGeom& cg, int N, int KN,
-                          int K_unpack, float alpha, float* d_y, hipStream_t st);
+                          int K_unpack, float alpha, float* d_y, hipStream_t st, const QuantOut& qo = QuantOut());
 
 
-// ---- ftnn_api.hip ----
-// the fp4 layer with weights expanded beforehand (d_wf: launch_mfma_expand(true, ...) of the packed rows);
-// d_p4 receives the quantised input: N*H*W*C_pack*32 bytes.  Arguments already validated.
+// ---- ftnn_api.hip ----  (arguments already validated)
+// The fp4 layer with weights expanded beforehand (d_wf: launch_mfma_expand(true, ...) of the packed rows).
+// d_x != null: the input is quantised into d_p4 (N*H*W*C_pack*32 bytes) first; d_x == null: d_p4 already
+// holds it (written by the previous layer through its QuantOut).  qo.mode != 0: d_y is not written.
 int conv_f4_expanded(int type, const float* d_x, const float* d_thr, const void* d_wf, int N, int C, int H,
                      int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride, int W_stride,
-                     float prelu_alpha, void* d_p4, float* d_y, hipStream_t st);
+                     float prelu_alpha, void* d_p4, float* d_y, hipStream_t st, const QuantOut& qo);
+// the vector-ALU layer; d_scratch as for ftnn_conv
+// (weights_prepared: for a few-channel layer d_qw already holds the re-packed rows of launch_dense_weights)
+int conv_valu(int type, const float* d_x, const float* d_thr, const int64_t* d_qw, int N, int C, int H, int W,
+              int KN, int KH, int KW, int H_pad, int W_pad, int H_stride, int W_stride, float prelu_alpha,
+              void* d_scratch, float* d_y, hipStream_t st, const QuantOut& qo, bool weights_prepared);
+// bytes of the fp4 layer's operand region (d_p4 above) for this shape, rounded up to 256: P4, or for a
+// few-channel layer the nibble pixels and dense rows
+int64_t conv_f4_operand_bytes(int N, int C, int H, int W, int KH, int KW, int OH, int OW);
+// words per row of the weights as the fp4 layer reads them (the dense re-packing shortens them)
+int conv_f4_weight_words(int C, int KH, int KW);
 
 }  // namespace ftnn

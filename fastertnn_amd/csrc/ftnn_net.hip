@@ -1,5 +1,13 @@
 // Chain of conv layers with device-resident activations (the reference's e2e mode,
 // src/timing_layers.c:182-207, without the per-layer host round trip).
+//
+// Between two layers the reference holds fp32 activations (its tnns_conv returns them and the next
+// call quantises them again).  Here a layer that feeds a layer on the fp4 matrix-core engine
+// quantises its own results in its epilogue, with the next layer's thresholds, and writes that
+// layer's operand (P4) directly: the fp32 tensor in between (e.g. 103 MB after a batch-32 stem)
+// is neither written nor read, and the next layer needs no quantise launch.  The values compared
+// against the thresholds are the same fp32 numbers, so the chain's output is unchanged.
+#include <algorithm>
 #include <new>
 #include <vector>
 
@@ -12,8 +20,9 @@ struct ftnn_net {
     std::vector<int> OH, OW;
     std::vector<float*> d_thr;       // per layer: batch copies of its threshold
     std::vector<void*> d_wf;         // per layer on the fp4 engine: its weights as matrix-core fragments
-    float* d_act[2] = {nullptr, nullptr};
-    void* d_scratch = nullptr;
+    float* d_act[2] = {nullptr, nullptr};   // fp32 activations between layers that need them
+    void* d_p4[2] = {nullptr, nullptr};     // quantised input of the fp4 layers, by layer parity
+    void* d_scratch = nullptr;              // work space of the vector-ALU layers
     int64_t out_elems = 0;
     // recorded graph and what it was recorded for
     hipGraphExec_t exec = nullptr;
@@ -28,19 +37,31 @@ using namespace ftnn;
 
 int enqueue_layers(ftnn_net* net, const float* d_x, float* d_y, hipStream_t st) {
     const int n = (int)net->layers.size();
-    const float* in = d_x;
+    const float* in = d_x;    // fp32 input of layer i (unused when p4_ready)
+    bool p4_ready = false;    // d_p4[i & 1] already holds layer i's quantised input
     for (int i = 0; i < n; i++) {
         const ftnn_layer_t& L = net->layers[i];
-        float* out = (i == n - 1) ? d_y : net->d_act[i & 1];
+        // the next layer takes a quantised hand-over if it is an fp4 layer that reads P4 (not a few-channel one)
+        const bool next_f4 = i + 1 < n && net->d_wf[i + 1] &&
+                             !dense_f4_applies(net->layers[i + 1].C, net->layers[i + 1].KH, net->layers[i + 1].KW);
+        QuantOut qo;
+        if (next_f4) {
+            const int nt = net->layers[i + 1].type;
+            qo.p4 = net->d_p4[(i + 1) & 1];
+            qo.thr = net->d_thr[i + 1];
+            qo.mode = (nt == kTNN || nt == kTBN) ? 1 : 2;
+        }
+        float* out = next_f4 ? nullptr : ((i == n - 1) ? d_y : net->d_act[i & 1]);
         int rc;
         if (net->d_wf[i])
-            rc = conv_f4_expanded(L.type, in, net->d_thr[i], net->d_wf[i], net->batch, L.C, L.H, L.W, L.KN, L.KH,
-                                  L.KW, L.pad, L.pad, L.stride, L.stride, L.prelu_alpha, net->d_scratch, out, st);
+            rc = conv_f4_expanded(L.type, p4_ready ? nullptr : in, net->d_thr[i], net->d_wf[i], net->batch, L.C, L.H,
+                                  L.W, L.KN, L.KH, L.KW, L.pad, L.pad, L.stride, L.stride, L.prelu_alpha,
+                                  net->d_p4[i & 1], out, st, qo);
         else
-            rc = ftnn_conv_engine(FTNN_ENGINE_VALU, L.type, in, net->d_thr[i], L.d_qw, net->batch, L.C, L.H, L.W,
-                                  L.KN, L.KH, L.KW, L.pad, L.pad, L.stride, L.stride, L.prelu_alpha,
-                                  net->d_scratch, out, st);
+            rc = conv_valu(L.type, in, net->d_thr[i], L.d_qw, net->batch, L.C, L.H, L.W, L.KN, L.KH, L.KW, L.pad,
+                           L.pad, L.stride, L.stride, L.prelu_alpha, net->d_scratch, out, st, qo, false);
         if (rc != FTNN_OK) return rc;
+        p4_ready = next_f4;
         in = out;
     }
     return FTNN_OK;
@@ -66,7 +87,6 @@ ftnn_net_t* ftnn_net_create(int batch, int n_layers, const ftnn_layer_t* layers)
         return nullptr;
     }
     net->batch = batch;
-    int64_t max_act = 0, max_scratch = 0;
     for (int i = 0; i < n_layers; i++) {
         const ftnn_layer_t& L = layers[i];
         const bool ok = L.type >= kTNN && L.type <= kBNN && L.C > 0 && L.H > 0 && L.W > 0 && L.KN > 0 &&
@@ -89,16 +109,31 @@ ftnn_net_t* ftnn_net_create(int batch, int n_layers, const ftnn_layer_t* layers)
         net->layers.push_back(L);
         net->OH.push_back(out_dim(L.H, L.pad, L.KH, L.stride));
         net->OW.push_back(out_dim(L.W, L.pad, L.KW, L.stride));
-        const int64_t out = (int64_t)batch * L.KN * net->OH[i] * net->OW[i];
-        if (i < n_layers - 1 && out > max_act) max_act = out;
-        const int64_t scr = ftnn_conv_scratch_bytes(L.type, batch, L.C, L.H, L.W, L.KN, L.KH, L.KW, L.pad, L.pad,
-                                                    L.stride, L.stride);
-        if (scr > max_scratch) max_scratch = scr;
-        net->out_elems = out;
+        net->out_elems = (int64_t)batch * L.KN * net->OH[i] * net->OW[i];
+    }
+    // engine of every layer, then the buffers the chain needs between them
+    std::vector<char> f4((size_t)n_layers, 0);
+    int64_t max_act = 0, max_scratch = 256, max_p4 = 0;
+    for (int i = 0; i < n_layers; i++) {
+        const ftnn_layer_t& L = layers[i];
+        f4[i] = ftnn_select_conv_engine(L.type, batch, L.C, L.H, L.W, L.KN, L.KH, L.KW, L.pad, L.pad, L.stride,
+                                        L.stride) == FTNN_ENGINE_MFMA_F4;
+        if (f4[i]) {
+            max_p4 = std::max(max_p4, conv_f4_operand_bytes(batch, L.C, L.H, L.W, L.KH, L.KW, net->OH[i], net->OW[i]));
+            if (i > 0 && dense_f4_applies(L.C, L.KH, L.KW))   // its input arrives as fp32
+                max_act = std::max(max_act, (int64_t)batch * L.C * L.H * L.W);
+        } else {
+            max_scratch = std::max(max_scratch, ftnn_conv_scratch_bytes(L.type, batch, L.C, L.H, L.W, L.KN, L.KH, L.KW,
+                                                                        L.pad, L.pad, L.stride, L.stride));
+            if (i > 0)   // its input arrives as fp32
+                max_act = std::max(max_act, (int64_t)batch * L.C * L.H * L.W);
+        }
     }
     bool good = hipMalloc(&net->d_scratch, (size_t)max_scratch) == hipSuccess;
     for (int b = 0; b < 2 && good && max_act > 0; b++)
         good = hipMalloc((void**)&net->d_act[b], (size_t)max_act * sizeof(float)) == hipSuccess;
+    for (int b = 0; b < 2 && good && max_p4 > 0; b++)
+        good = hipMalloc(&net->d_p4[b], (size_t)max_p4) == hipSuccess;
     std::vector<float> host((size_t)batch);
     for (int i = 0; i < n_layers && good; i++) {
         float* d = nullptr;
@@ -112,15 +147,22 @@ ftnn_net_t* ftnn_net_create(int batch, int n_layers, const ftnn_layer_t* layers)
     net->d_wf.assign((size_t)n_layers, nullptr);
     for (int i = 0; i < n_layers && good; i++) {
         const ftnn_layer_t& L = layers[i];
-        if (ftnn_select_conv_engine(L.type, batch, L.C, L.H, L.W, L.KN, L.KH, L.KW, L.pad, L.pad, L.stride,
-                                    L.stride) != FTNN_ENGINE_MFMA_F4)
-            continue;
-        const int Kw = round4(cpack_of(L.C) * L.KH * L.KW);
+        if (!f4[i]) continue;
+        const int Kw = conv_f4_weight_words(L.C, L.KH, L.KW);
+        const bool wt = L.type == kTNN || L.type == kBTN;
         good = hipMalloc(&net->d_wf[i], (size_t)mfma_fragment_bytes(true, L.KN, Kw)) == hipSuccess;
         if (!good) break;
-        good = launch_mfma_expand(true, L.type == kTNN || L.type == kBTN, L.d_qw, L.KN, Kw, net->d_wf[i], nullptr) ==
-                   hipSuccess &&
+        const int64_t* rows = L.d_qw;
+        void* d_wd = nullptr;
+        if (dense_f4_applies(L.C, L.KH, L.KW)) {   // few channels: the weights take the dense re-packing first
+            good = hipMalloc(&d_wd, (size_t)L.KN * Kw * (wt ? 16 : 8)) == hipSuccess &&
+                   launch_dense_weights(wt, L.d_qw, L.KN, L.C, L.KH, L.KW, static_cast<int64_t*>(d_wd), nullptr) ==
+                       hipSuccess;
+            rows = static_cast<const int64_t*>(d_wd);
+        }
+        good = good && launch_mfma_expand(true, wt, rows, L.KN, Kw, net->d_wf[i], nullptr) == hipSuccess &&
                hipStreamSynchronize(nullptr) == hipSuccess;
+        if (d_wd) (void)hipFree(d_wd);
     }
     if (!good) {
         fail(FTNN_ENOMEM, "device allocation for the layer chain failed");
@@ -138,6 +180,8 @@ void ftnn_net_destroy(ftnn_net_t* net) {
         if (p) (void)hipFree(p);
     for (int b = 0; b < 2; b++)
         if (net->d_act[b]) (void)hipFree(net->d_act[b]);
+    for (int b = 0; b < 2; b++)
+        if (net->d_p4[b]) (void)hipFree(net->d_p4[b]);
     if (net->d_scratch) (void)hipFree(net->d_scratch);
     delete net;
 }

@@ -294,10 +294,14 @@ struct ConvFrag {
     bool in[2];   // x[b] holds a real input pixel (else the padding value replaces it)
 };
 
-template <bool ABIN, int S>
+// ABIN: binary activations (padding value +1).  FORM0: the TNN form of PReLU, "f <= 0 -> f *= alpha"
+// (mm_p2_final_tnn_avx2.c:204-208), else "r >= 0 ? r : alpha * r" (mm_p2_final_tbn_avx2.c:73).
+// QMODE: 0 = fp32 NCHW result, 1 / 2 = ternary / binary hand-over to the next layer (QuantOut).
+// All three are compile-time so that the per-element epilogue carries no selects for them.
+template <bool ABIN, bool FORM0, int QMODE, int S>
 __global__ __launch_bounds__(256) void k_conv_f4(const uint4* __restrict__ P4, const uint4* __restrict__ Wf,
                                                  float* __restrict__ Y, int M, int KN, int OHW, int KB,
-                                                 int bias, int form, float alpha, FastDiv dOHW, ConvGeom cg) {
+                                                 int bias, float alpha, FastDiv dOHW, ConvGeom cg, QuantOut qo) {
     constexpr int NB = 3;                 // register sets of fragments: NB - 1 steps of loads in flight
     constexpr int PUB = 4 - 4 / S;        // blocks a wavefront hands to the others of its tile
     __shared__ float4 red[S > 1 ? 4 * PUB * 4 * 64 : 1];   // [wavefront][slot][e / 4][lane]
@@ -426,7 +430,6 @@ __global__ __launch_bounds__(256) void k_conv_f4(const uint4* __restrict__ P4, c
         });
         __syncthreads();
     }
-    const bool le_form = form == 0;
     for_blocks([&](auto blk_tag) {
         constexpr int BLK = decltype(blk_tag)::value;
         if (BLK % S == ks) {
@@ -453,16 +456,61 @@ __global__ __launch_bounds__(256) void k_conv_f4(const uint4* __restrict__ P4, c
             const int q = px0 + 32 * b + lr;
             const uint32_t qc = (uint32_t)min(q, M - 1);
             const uint32_t img = fastdiv(qc, dOHW);
-            float* yq = Y + (size_t)img * KN * OHW + (qc - img * (uint32_t)OHW);
+            const uint32_t pix = qc - img * (uint32_t)OHW;
+            // r = acc - bias: both are integers below 2^24 in fp32, and so is their difference
+            const float fbias = (float)bias;
+            float vals[16];
 #pragma unroll
             for (int e = 0; e < 16; e++) {
-                const int p = kn0 + 32 * a + 8 * (e >> 2) + 4 * h + (e & 3);
-                const int r = (int)mine[e] - bias;
-                const float fr = (float)r;
+                const float fr = mine[e] - fbias;
                 // form 0: scale when f <= 0 (a zero becomes 0 * alpha); form 1: scale when r < 0
-                const bool scale = le_form ? (fr <= 0.0f) : (r < 0);
-                const float fv = scale ? fr * alpha : fr;
-                if (q < M && p < KN) yq[(size_t)p * OHW] = fv;
+                const bool scale = FORM0 ? (fr <= 0.0f) : (fr < 0.0f);
+                vals[e] = scale ? fr * alpha : fr;
+            }
+            if constexpr (QMODE == 0) {
+                float* yq = Y + ((size_t)img * KN + kn0 + 32 * a + 4 * h) * OHW + pix;
+                if (q < M) {
+                    if (kn0 + 32 * a + 32 <= KN) {   // whole block inside: no per-kernel checks
+#pragma unroll
+                        for (int e = 0; e < 16; e++) yq[(size_t)((8 * (e >> 2) + (e & 3)) * OHW)] = vals[e];
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 16; e++) {
+                            const int p = kn0 + 32 * a + 8 * (e >> 2) + 4 * h + (e & 3);
+                            if (p < KN) yq[(size_t)((8 * (e >> 2) + (e & 3)) * OHW)] = vals[e];
+                        }
+                    }
+                }
+            } else {
+                // Hand-over to an fp4 layer.  Registers 4g .. 4g+3 of this lane are kernels
+                // 8g + 4h + {0..3} of the block: half of nibble dword g of the pixel; the other
+                // half sits in lane ^ 32.  Lane h ends up with dwords 2h and 2h + 1 of the
+                // block's 16 bytes, i.e. bytes 16a + 8h .. + 8 of the pixel's 64-channel word.
+                const float t = qo.thr[img];
+                constexpr bool tern = QMODE == 1;
+                const bool inside = kn0 + 32 * a + 32 <= KN;   // uniform: no per-kernel checks then
+                uint32_t half[4];
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    half[g] = 0u;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const bool live = inside || kn0 + 32 * a + 8 * g + 4 * h + i < KN;
+                        half[g] |= quant_nibble(vals[4 * g + i], t, tern, live) << (4 * i);
+                    }
+                }
+                const uint32_t send = h ? (half[0] | (half[1] << 16)) : (half[2] | (half[3] << 16));
+                const uint32_t recv = (uint32_t)__shfl_xor((int)send, 32, 64);
+                uint2 out;
+                if (h == 0) {
+                    out.x = half[0] | (recv << 16);
+                    out.y = half[1] | (recv & 0xffff0000u);
+                } else {
+                    out.x = (recv & 0xffffu) | (half[2] << 16);
+                    out.y = (recv >> 16) | (half[3] << 16);
+                }
+                const size_t word = ((size_t)img * gridDim.y + blockIdx.y) * OHW + pix;
+                if (q < M) *reinterpret_cast<uint2*>(static_cast<unsigned char*>(qo.p4) + word * 32 + 16 * a + 8 * h) = out;
             }
         }
     });
@@ -526,13 +574,12 @@ hipError_t launch_mfma_gemm(bool f4, int type, const void* d_af, const void* d_b
 }
 
 hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const ConvGeom& cg, int N, int KN,
-                          int K_unpack, float alpha, float* d_y, hipStream_t st) {
+                          int K_unpack, float alpha, float* d_y, hipStream_t st, const QuantOut& qo) {
     const int OHW = cg.OH * cg.OW;
     const int64_t M = (int64_t)N * OHW;
     const int KB = round4(cg.K);
     // BNN: the channel lanes past C are +1 in both operands (see launch_mfma_gemm); padding words are skipped
     const int bias = type == kBNN ? 64 * cg.K - K_unpack : 0;
-    const int form = type == kTNN ? 0 : 1;
     // K split: enough wavefronts to occupy the chip's 1024 SIMDs, but no exchange where the tiles
     // alone do that (a tile = 64 kernels x 64 pixels)
     const int64_t tiles = ((M + 63) / 64) * ((KN + 63) / 64);
@@ -544,20 +591,37 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
     const uint4* P4 = static_cast<const uint4*>(d_p4);
     const uint4* Wf = static_cast<const uint4*>(d_wf);
     const FastDiv dOHW = make_fastdiv((uint32_t)OHW);
-    const bool abin = type == kBTN || type == kBNN;
-#define FTNN_CONV(S_)                                                                                            \
-    if (split == S_) {                                                                                           \
-        if (abin)                                                                                                \
-            hipLaunchKernelGGL((k_conv_f4<true, S_>), grid, dim3(256), 0, st, P4, Wf, d_y, (int)M, KN, OHW, KB,  \
-                               bias, form, alpha, dOHW, cg);                                                     \
-        else                                                                                                     \
-            hipLaunchKernelGGL((k_conv_f4<false, S_>), grid, dim3(256), 0, st, P4, Wf, d_y, (int)M, KN, OHW, KB, \
-                               bias, form, alpha, dOHW, cg);                                                     \
-        return hipGetLastError();                                                                                \
-    }
-    FTNN_CONV(1) FTNN_CONV(2) FTNN_CONV(4)
-#undef FTNN_CONV
-    return hipErrorInvalidValue;
+    // The kernel's hand-counted loads write registers behind the compiler's back; that is only
+    // sound while none of its registers live in scratch memory, which is checked once per variant.
+    auto launch = [&](auto kern) -> hipError_t {
+        static const hipError_t sound = [&]() {
+            hipFuncAttributes attr;
+            hipError_t e = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(kern));
+            if (e == hipSuccess && attr.localSizeBytes != 0) e = hipErrorLaunchFailure;
+            return e;
+        }();
+        if (sound != hipSuccess) return sound;
+        hipLaunchKernelGGL(kern, grid, dim3(256), 0, st, P4, Wf, d_y, (int)M, KN, OHW, KB, bias, alpha, dOHW, cg, qo);
+        return hipGetLastError();
+    };
+    // kernel variant: activation kind and PReLU form follow the type, then hand-over mode and split
+    auto by_split = [&](auto abin, auto form0, auto qmode) -> hipError_t {
+        constexpr bool A = decltype(abin)::value, F = decltype(form0)::value;
+        constexpr int Q = decltype(qmode)::value;
+        if (split == 1) return launch(k_conv_f4<A, F, Q, 1>);
+        if (split == 2) return launch(k_conv_f4<A, F, Q, 2>);
+        if (split == 4) return launch(k_conv_f4<A, F, Q, 4>);
+        return hipErrorInvalidValue;
+    };
+    auto by_mode = [&](auto abin, auto form0) -> hipError_t {
+        if (qo.mode == 0) return by_split(abin, form0, std::integral_constant<int, 0>{});
+        if (qo.mode == 1) return by_split(abin, form0, std::integral_constant<int, 1>{});
+        if (qo.mode == 2) return by_split(abin, form0, std::integral_constant<int, 2>{});
+        return hipErrorInvalidValue;
+    };
+    if (type == kTNN) return by_mode(std::false_type{}, std::true_type{});
+    if (type == kTBN) return by_mode(std::false_type{}, std::false_type{});
+    return by_mode(std::true_type{}, std::false_type{});   // BTN, BNN
 }
 
 hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* d_b, int64_t M, int OHW,

@@ -109,7 +109,7 @@ template <int MODE, int TM, int TN, int GC, bool IMPL, bool TR = false>
 __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
                                             const uint32_t* __restrict__ B,
                                             float* __restrict__ Y, int M, int KN, int OHW, int G,
-                                            int K_unpack, float alpha, FastDiv dOHW, ConvGeom cg) {
+                                            int K_unpack, float alpha, FastDiv dOHW, ConvGeom cg, QuantOut qo) {
     using T = Traits<MODE>;
     constexpr int BM = 64 * TM;
     constexpr int AG = T::kAGroup, BG = T::kBGroup;
@@ -318,7 +318,21 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
     for (int a = 0; a < TM; a++) {
         const int64_t i = row0 + lane + 64 * a;
         if (i < M) {
-            if (TR) {   // consecutive lanes write consecutive floats of one output row
+            if (!TR && qo.mode != 0) {
+                // hand-over to an fp4 layer: this lane's TN kernels are TN consecutive nibbles of one pixel
+                const uint32_t img = fastdiv((uint32_t)i, dOHW);
+                const uint32_t pix = (uint32_t)i - img * (uint32_t)OHW;
+                const float t = qo.thr[img];
+                uint32_t dw = 0u;
+#pragma unroll
+                for (int b = 0; b < TN; b++)
+                    dw |= quant_nibble(finish(a, b), t, qo.mode == 1, col0 + b < KN) << (4 * b);
+                const size_t word = ((size_t)img * ((KN + 63) / 64) + (col0 >> 6)) * OHW + pix;
+                unsigned char* dst = static_cast<unsigned char*>(qo.p4) + word * 32 + ((col0 & 63) >> 1);
+                if (TN == 8) *reinterpret_cast<uint32_t*>(dst) = dw;
+                else if (TN == 4) *reinterpret_cast<unsigned short*>(dst) = (unsigned short)dw;
+                else *dst = (unsigned char)dw;
+            } else if (TR) {   // consecutive lanes write consecutive floats of one output row
 #pragma unroll
                 for (int b = 0; b < TN; b++) {
                     const int j = col0 + b;
@@ -346,18 +360,21 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
 
 template <int MODE, int TM, int TN, int GC, bool IMPL, bool TR>
 hipError_t launch_cfg(const uint32_t* A, const uint32_t* B, float* Y, int64_t M, int KN, int OHW,
-                      int G, int K_unpack, float alpha, const ConvGeom& cg, hipStream_t st) {
+                      int G, int K_unpack, float alpha, const ConvGeom& cg, hipStream_t st, const QuantOut& qo) {
     const int64_t gx = (M + 64 * TM - 1) / (64 * TM);
-    const int64_t gy = (KN + 4 * TN - 1) / (4 * TN);
+    // with a quantised hand-over every 64-channel word that holds a kernel is written in full
+    const int cols = qo.mode != 0 ? (KN + 63) / 64 * 64 : KN;
+    const int64_t gy = (cols + 4 * TN - 1) / (4 * TN);
     if (gx > 0x7fffffffLL || gy > 65535) return hipErrorInvalidValue;
     hipLaunchKernelGGL((k_mm<MODE, TM, TN, GC, IMPL, TR>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
-                       A, B, Y, (int)M, KN, OHW, G, K_unpack, alpha, make_fastdiv((uint32_t)OHW), cg);
+                       A, B, Y, (int)M, KN, OHW, G, K_unpack, alpha, make_fastdiv((uint32_t)OHW), cg, qo);
     return hipGetLastError();
 }
 
 template <int MODE, bool IMPL, bool TR = false>
 hipError_t launch_mode(const uint32_t* A, const uint32_t* B, float* Y, int64_t M, int KN, int OHW,
-                       int G, int K_unpack, float alpha, const ConvGeom& cg, hipStream_t st) {
+                       int G, int K_unpack, float alpha, const ConvGeom& cg, hipStream_t st,
+                       const QuantOut& qo = QuantOut()) {
     // Tile choice (measured on MI355X): 128 x 32 tiles once they give each of the 256 CUs
     // a dozen workgroups; layer-sized problems are one or two waves of workgroups, where
     // smaller tiles finish sooner.
@@ -369,20 +386,20 @@ hipError_t launch_mode(const uint32_t* A, const uint32_t* B, float* Y, int64_t M
         int tm = 0, tn = 0;
         sscanf(force, "%d,%d", &tm, &tn);
 #define FTNN_TRY(TM_, TN_) \
-    if (tm == TM_ && tn == TN_) return launch_cfg<MODE, TM_, TN_, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+    if (tm == TM_ && tn == TN_) return launch_cfg<MODE, TM_, TN_, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
         FTNN_TRY(2, 8) FTNN_TRY(1, 8) FTNN_TRY(1, 4) FTNN_TRY(1, 2)
 #undef FTNN_TRY
     }
-    if (wgs(2, 8) >= 3072) return launch_cfg<MODE, 2, 8, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
-    if (wgs(1, 8) >= 1536) return launch_cfg<MODE, 1, 8, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
-    if (wgs(1, 4) >= 2048) return launch_cfg<MODE, 1, 4, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
-    return launch_cfg<MODE, 1, 2, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+    if (wgs(2, 8) >= 3072) return launch_cfg<MODE, 2, 8, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
+    if (wgs(1, 8) >= 1536) return launch_cfg<MODE, 1, 8, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
+    if (wgs(1, 4) >= 2048) return launch_cfg<MODE, 1, 4, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
+    return launch_cfg<MODE, 1, 2, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
 }
 
 }  // namespace
 
 hipError_t launch_mm(int type, const int64_t* d_a, const int64_t* d_b, int64_t M, int OHW, int KN,
-                     int Kw, int K_unpack, float alpha, float* d_y, hipStream_t st) {
+                     int Kw, int K_unpack, float alpha, float* d_y, hipStream_t st, const QuantOut& qo) {
     const uint32_t* A = reinterpret_cast<const uint32_t*>(d_a);
     const uint32_t* B = reinterpret_cast<const uint32_t*>(d_b);
     const int G = Kw / 4;
@@ -393,29 +410,29 @@ hipError_t launch_mm(int type, const int64_t* d_a, const int64_t* d_b, int64_t M
     // come from the TBN form with the operands exchanged (ternary B along the lanes, binary A in
     // scalar registers) and the result stored transposed; both types share one PReLU form
     // (src/tnns/mm_p2_final_tbn_avx2.c:72-73, src/tnns/mm_p2_final_btn_avx2.c:72-73).
-    if (type == kBTN && OHW == 1 && KN >= 64 && M <= 0x7fffffff)
-        return launch_mode<kTBN, false, true>(B, A, d_y, KN, (int)M, 1, G, K_unpack, alpha, cg, st);
+    if (type == kBTN && OHW == 1 && KN >= 64 && M <= 0x7fffffff && qo.mode == 0)
+        return launch_mode<kTBN, false, true>(B, A, d_y, KN, (int)M, 1, G, K_unpack, alpha, cg, st, qo);
     switch (type) {
-        case kTNN: return launch_mode<kTNN, false>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
-        case kTBN: return launch_mode<kTBN, false>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
-        case kBTN: return launch_mode<kBTN, false>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
-        case kBNN: return launch_mode<kBNN, false>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+        case kTNN: return launch_mode<kTNN, false>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
+        case kTBN: return launch_mode<kTBN, false>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
+        case kBTN: return launch_mode<kBTN, false>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
+        case kBNN: return launch_mode<kBNN, false>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
     }
     return hipErrorInvalidValue;
 }
 
 hipError_t launch_mm_implicit(int type, const void* d_p, const int64_t* d_b, const ConvGeom& cg, int N,
-                              int KN, int K_unpack, float alpha, float* d_y, hipStream_t st) {
+                              int KN, int K_unpack, float alpha, float* d_y, hipStream_t st, const QuantOut& qo) {
     const uint32_t* A = static_cast<const uint32_t*>(d_p);
     const uint32_t* B = reinterpret_cast<const uint32_t*>(d_b);
     const int OHW = cg.OH * cg.OW;
     const int64_t M = (int64_t)N * OHW;
     const int G = round4(cg.K) / 4;
     switch (type) {
-        case kTNN: return launch_mode<kTNN, true>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
-        case kTBN: return launch_mode<kTBN, true>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
-        case kBTN: return launch_mode<kBTN, true>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
-        case kBNN: return launch_mode<kBNN, true>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st);
+        case kTNN: return launch_mode<kTNN, true>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
+        case kTBN: return launch_mode<kTBN, true>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
+        case kBTN: return launch_mode<kBTN, true>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
+        case kBNN: return launch_mode<kBNN, true>(A, B, d_y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
     }
     return hipErrorInvalidValue;
 }

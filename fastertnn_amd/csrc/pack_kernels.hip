@@ -304,6 +304,88 @@ __global__ __launch_bounds__(256) void k_dense_rows(const unsigned long long* __
     }
 }
 
+// ---- the same re-packing for the fp4 matrix-core layer kernel (C <= 8) ----
+// k_quantize_nib: one dword per pixel, nibble c = channel c as E2M1 (0x2 / 0x0 / 0xA), channels past C
+// as the padding lane of the type (ternary 0, binary +1).
+template <bool TERN>
+__global__ __launch_bounds__(256) void k_quantize_nib(const float* __restrict__ x, const float* __restrict__ thr,
+                                                      int C, int HW, uint32_t* __restrict__ Pq) {
+    const int p = blockIdx.x * 256 + threadIdx.x, n = blockIdx.y;
+    if (p >= HW) return;
+    const float t = thr[n];
+    const float* xp = x + (size_t)n * C * HW + p;
+    uint32_t dw = 0u;
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+        const float v = c < C ? xp[(size_t)c * HW] : 0.0f;
+        uint32_t nib;
+        if (TERN) nib = c < C ? (v < -t ? 0xAu : (v > t ? 0x2u : 0x0u)) : 0x0u;
+        else nib = c < C ? (v < t ? 0xAu : 0x2u) : 0x2u;
+        dw |= nib << (4 * c);
+    }
+    Pq[(size_t)n * HW + p] = dw;
+}
+
+// k_dense_rows_f4: one work-item per (output pixel, dense word d) strings the C nibbles of taps
+// d*T .. d*T + T - 1 together (lane (tap % T)*C + c, as in k_dense_rows), then the lanes left over,
+// 64 lanes = 32 bytes in all, and the block writes its 8 KiB through LDS in one contiguous piece.
+// Taps outside the image, taps past KH*KW and left-over lanes hold the padding lane of the type.
+// Output = the fp4 layer kernel's operand for a 1x1 layer over the output pixels with Kd words per
+// pixel: A4[n][d][pixel][32 bytes].
+template <bool TERN>
+__global__ __launch_bounds__(256) void k_dense_rows_f4(const uint32_t* __restrict__ Pq, int C, int T, int H, int W,
+                                                       int OHW, int OW, int KW, int taps, int Kd, int H_pad,
+                                                       int W_pad, int H_stride, int W_stride, FastDiv dOW,
+                                                       FastDiv dKW, uint32_t* __restrict__ A4) {
+    __shared__ uint32_t s_out[256 * 9];
+    const int pix = blockIdx.x * 256 + threadIdx.x, d = blockIdx.y, n = blockIdx.z;
+    const uint32_t padv = TERN ? 0u : 0x22222222u;
+    if (pix < OHW) {
+        const int oh = (int)fastdiv((uint32_t)pix, dOW), ow = pix - oh * OW;
+        const int ih0 = oh * H_stride - H_pad, iw0 = ow * W_stride - W_pad;
+        const uint32_t* img = Pq + (size_t)n * H * W;
+        const uint32_t cmask = C >= 8 ? 0xffffffffu : ((1u << (4 * C)) - 1u);
+        const int tap0 = d * T;
+        int kh = (int)fastdiv((uint32_t)tap0, dKW), kw = tap0 - kh * KW;
+        unsigned long long cur = 0ull;
+        int pos = 0, k = 0;
+        uint32_t* mine = s_out + threadIdx.x * 9;
+        for (int j = 0; j <= T; j++) {
+            uint32_t v;
+            int bits;
+            if (j < T) {
+                const int ih = ih0 + kh, iw = iw0 + kw;
+                const bool in = tap0 + j < taps && (unsigned)ih < (unsigned)H && (unsigned)iw < (unsigned)W;
+                v = (in ? img[ih * W + iw] : padv) & cmask;
+                bits = 4 * C;
+                if (++kw == KW) {
+                    kw = 0;
+                    kh++;
+                }
+            } else {   // the lanes left over after T taps
+                bits = 4 * (64 - T * C);
+                v = bits ? (padv & ((1u << bits) - 1u)) : 0u;   // bits < 32: fewer than C <= 8 lanes are left
+            }
+            cur |= (unsigned long long)v << pos;
+            pos += bits;
+            if (pos >= 32) {
+                mine[k++] = (uint32_t)cur;
+                cur >>= 32;
+                pos -= 32;
+            }
+        }
+    }
+    __syncthreads();
+    // 256 pixels x 8 dwords, contiguous in A4 for this (n, d)
+    const int pix0 = blockIdx.x * 256;
+    uint32_t* dst = A4 + (((size_t)n * Kd + d) * OHW + pix0) * 8;
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+        const int e = it * 256 + threadIdx.x;
+        if (pix0 + (e >> 3) < OHW) dst[e] = s_out[(e >> 3) * 9 + (e & 7)];
+    }
+}
+
 // weights: one work-item per (kernel, dense word); source rows are the reference's packed rows
 // with C_pack = 1 (word index = tap)
 template <bool TERN>
@@ -365,6 +447,35 @@ hipError_t launch_dense_rows(bool ternary, const void* d_p, int N, int C, int H,
     else
         hipLaunchKernelGGL((k_dense_rows<false>), dim3(blocks), dim3(256), 0, st, P, C, T, H, W, OH, OW, kW,
                            kH * kW, Kd, Kdw, H_pad, W_pad, H_stride, W_stride, total, out);
+    return hipGetLastError();
+}
+
+bool dense_f4_applies(int C, int KH, int KW) { return C <= 8 && dense_applies(C, KH, KW, nullptr, nullptr); }
+
+int64_t dense_f4_pq_bytes(int N, int H, int W) { return ((int64_t)N * H * W * 4 + 255) / 256 * 256; }
+
+hipError_t launch_dense_rows_f4(bool ternary, const float* d_x, const float* d_thr, int N, int C, int H, int W,
+                                int H_pad, int W_pad, int kH, int kW, int H_stride, int W_stride, void* d_pq,
+                                void* d_a4, hipStream_t st) {
+    int T, Kd;
+    dense_applies(C, kH, kW, &T, &Kd);
+    const int OH = out_dim(H, H_pad, kH, H_stride), OW = out_dim(W, W_pad, kW, W_stride);
+    const int HW = H * W, OHW = OH * OW;
+    if (N > 65535 || Kd > 65535) return hipErrorInvalidValue;
+    uint32_t* Pq = static_cast<uint32_t*>(d_pq);
+    uint32_t* A4 = static_cast<uint32_t*>(d_a4);
+    dim3 gq((HW + 255) / 256, N), gr((OHW + 255) / 256, Kd, N);
+    if (ternary) {
+        hipLaunchKernelGGL((k_quantize_nib<true>), gq, dim3(256), 0, st, d_x, d_thr, C, HW, Pq);
+        hipLaunchKernelGGL((k_dense_rows_f4<true>), gr, dim3(256), 0, st, Pq, C, T, H, W, OHW, OW, kW, kH * kW, Kd,
+                           H_pad, W_pad, H_stride, W_stride, make_fastdiv((uint32_t)OW), make_fastdiv((uint32_t)kW),
+                           A4);
+    } else {
+        hipLaunchKernelGGL((k_quantize_nib<false>), gq, dim3(256), 0, st, d_x, d_thr, C, HW, Pq);
+        hipLaunchKernelGGL((k_dense_rows_f4<false>), gr, dim3(256), 0, st, Pq, C, T, H, W, OHW, OW, kW, kH * kW, Kd,
+                           H_pad, W_pad, H_stride, W_stride, make_fastdiv((uint32_t)OW), make_fastdiv((uint32_t)kW),
+                           A4);
+    }
     return hipGetLastError();
 }
 

@@ -44,6 +44,10 @@ _L.ftnn_conv_scratch_bytes.argtypes = [C.c_int] * 12
 _L.ftnn_conv.argtypes = [C.c_int, _vp, _vp, _vp] + [C.c_int] * 11 + [C.c_float, _vp, _vp, _vp]
 _L.ftnn_conv_engine.argtypes = [C.c_int, C.c_int, _vp, _vp, _vp] + [C.c_int] * 11 + [C.c_float, _vp, _vp, _vp]
 _L.ftnn_select_conv_engine.argtypes = [C.c_int] * 12
+_L.ftnn_conv_weights_bytes.restype = C.c_int64
+_L.ftnn_conv_weights_bytes.argtypes = [C.c_int] * 5
+_L.ftnn_conv_prepare_weights.argtypes = [C.c_int, _vp] + [C.c_int] * 4 + [_vp, _vp]
+_L.ftnn_conv_prepared.argtypes = [C.c_int, _vp, _vp, _vp] + [C.c_int] * 11 + [C.c_float, _vp, _vp, _vp]
 _L.ftnn_pack_weights.argtypes = [C.c_int, _vp, _vp] + [C.c_int] * 4 + [_vp, _vp]
 _L.ftnn_pack_gemm_operand.argtypes = [_vp, C.c_int, C.c_int, _vp, _vp]
 for _n in ("t2r_p2_opt", "b2r"):
@@ -62,7 +66,8 @@ EXPORTS = ("tnns_conv", "tnns_gemm", "t2r_p2_opt", "b2r", "mm_tnn", "mm_tbn", "m
            "ftnn_pack_scratch_bytes", "ftnn_quantize_im2row", "ftnn_mm", "ftnn_conv",
            "ftnn_pack_weights", "ftnn_pack_gemm_operand", "ftnn_select_engine", "ftnn_mm_scratch_bytes",
            "ftnn_mm_engine", "ftnn_expand_bytes", "ftnn_expand_rows", "ftnn_mm_expanded",
-           "ftnn_conv_scratch_bytes", "ftnn_conv_engine", "ftnn_select_conv_engine", "ftnn_net_create", "ftnn_net_destroy", "ftnn_net_output_elems", "ftnn_net_run")
+           "ftnn_conv_scratch_bytes", "ftnn_conv_engine", "ftnn_select_conv_engine",
+           "ftnn_conv_weights_bytes", "ftnn_conv_prepare_weights", "ftnn_conv_prepared", "ftnn_net_create", "ftnn_net_destroy", "ftnn_net_output_elems", "ftnn_net_run")
 
 ENGINE_AUTO, ENGINE_VALU, ENGINE_MFMA_I8, ENGINE_MFMA_F4 = 0, 1, 2, 3
 ENGINE_NAMES = {ENGINE_VALU: "valu", ENGINE_MFMA_I8: "mfma_i8", ENGINE_MFMA_F4: "mfma_f4"}
@@ -202,6 +207,32 @@ def conv(typ, x, thr, qw, kn, kh, kw, pad, stride, alpha, scratch=None, out=None
     args = (typ, _dev(x, torch.float32), _dev(thr, torch.float32), _dev(qw), n, c, h, w, kn, kh, kw, pad, pad,
             stride, stride, alpha, _dev(scratch), _dev(out, torch.float32), _stream())
     _check(_L.ftnn_conv(*args) if engine == ENGINE_AUTO else _L.ftnn_conv_engine(engine, *args))
+    return out
+
+
+def prepare_conv_weights(typ, qw, c, kn, kh, kw):
+    """ftnn_conv_prepare_weights: the packed rows in the form the layer's engine reads (once per layer)."""
+    import torch
+    out = torch.empty(int(_L.ftnn_conv_weights_bytes(typ, c, kn, kh, kw)), dtype=torch.uint8, device=qw.device)
+    _check(_L.ftnn_conv_prepare_weights(typ, _dev(qw), c, kn, kh, kw, _dev(out), _stream()))
+    return out
+
+
+def conv_prepared(typ, x, thr, prepared, kn, kh, kw, pad, stride, alpha, scratch=None, out=None):
+    """ftnn_conv_prepared: one conv layer with weights from prepare_conv_weights."""
+    import torch
+    n, c, h, w = x.shape
+    oh, ow = out_dim(h, pad, kh, stride), out_dim(w, pad, kw, stride)
+    if oh <= 0 or ow <= 0:
+        raise FtnnError("kernel larger than padded input")
+    if scratch is None:
+        scratch = torch.empty(conv_scratch_bytes(typ, n, c, h, w, kn, kh, kw, pad, stride), dtype=torch.uint8,
+                              device=x.device)
+    if out is None:
+        out = torch.empty((n, kn, oh, ow), dtype=torch.float32, device=x.device)
+    _check(_L.ftnn_conv_prepared(typ, _dev(x, torch.float32), _dev(thr, torch.float32), _dev(prepared), n, c, h, w,
+                                 kn, kh, kw, pad, pad, stride, stride, alpha, _dev(scratch),
+                                 _dev(out, torch.float32), _stream()))
     return out
 
 

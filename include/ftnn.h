@@ -221,6 +221,21 @@ FTNN_API int ftnn_conv_engine(int engine, int type, const float *d_x, const floa
                               void *stream);
 
 /*
+ * Weights prepared once per layer (no counterpart in the reference, whose packed rows are final):
+ * ftnn_conv_prepare_weights turns the packed rows of ftnn_pack_weights / the reference's
+ * quantized_kernel_packing2 into the form the layer's engine reads -- matrix-core fragments, or
+ * the dense re-packing of a few-channel layer -- so that ftnn_conv_prepared does not repeat that
+ * work on every call.  d_prepared: ftnn_conv_weights_bytes() bytes, 16-byte aligned.  Result and
+ * scratch of ftnn_conv_prepared are those of ftnn_conv.
+ */
+FTNN_API int64_t ftnn_conv_weights_bytes(int type, int C, int KN, int KH, int KW);
+FTNN_API int ftnn_conv_prepare_weights(int type, const int64_t *d_qw, int C, int KN, int KH, int KW,
+                                       void *d_prepared, void *stream);
+FTNN_API int ftnn_conv_prepared(int type, const float *d_x, const float *d_thr, const void *d_prepared, int N,
+                                int C, int H, int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride,
+                                int W_stride, float prelu_alpha, void *d_scratch, float *d_y, void *stream);
+
+/*
  * A chain of conv layers with device-resident activations: the e2e mode of the reference's
  * layer driver (src/timing_layers.c:182-207 feeds each layer's output to the next one), here
  * without the host round trip per layer.  All device memory (two activation buffers, the

@@ -104,11 +104,14 @@ def test_engine_selection_and_scratch_sizes_need_no_device():
     assert lib.pack_scratch_bytes(2, 64, 8, 8, 1) == 2 * 8 * 8 * 16
     assert lib.conv_scratch_bytes(0, 2, 64, 8, 8, 16, 3, 3, 1, 1) == 2 * 8 * 8 * 32 + 1 * 12 * 1024
     valu_dense = 2 * 32 * 32 * 16 + 2 * 16 * 16 * 4 * 16 + 16 * 4 * 16
-    fp4 = 2 * 32 * 32 * 32 + 1 * 52 * 1024
-    assert lib.conv_scratch_bytes(0, 2, 3, 32, 32, 16, 7, 7, 3, 2) == max(valu_dense, fp4)
+    # fp4 with C <= 8: a nibble dword per input pixel, 32 bytes per output pixel and dense word, fragments and
+    # re-packed rows of the weights
+    fp4_dense = 2 * 32 * 32 * 4 + 2 * 16 * 16 * 3 * 32 + 1 * 4 * 1024 + 16 * 4 * 16
+    assert lib.conv_scratch_bytes(0, 2, 3, 32, 32, 16, 7, 7, 3, 2) == max(valu_dense, fp4_dense)
     # layer engine: fp4 wherever the dense re-packing does not apply and fp32 accumulation stays exact
     assert lib.select_conv_engine(0, 1, 256, 56, 56, 256, 3, 3, 1, 1) == lib.ENGINE_MFMA_F4
-    assert lib.select_conv_engine(0, 32, 3, 224, 224, 64, 7, 7, 3, 2) == lib.ENGINE_VALU
+    assert lib.select_conv_engine(0, 32, 3, 224, 224, 64, 7, 7, 3, 2) == lib.ENGINE_MFMA_F4   # dense re-packing, C <= 8
+    assert lib.select_conv_engine(0, 4, 16, 20, 20, 64, 3, 3, 1, 1) == lib.ENGINE_VALU         # dense re-packing, C > 8
 
 
 def test_missing_library_is_an_import_error(tmp_path):

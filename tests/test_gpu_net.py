@@ -20,10 +20,29 @@ STACK = [
 ]
 
 
-def build(hip, oracle, batch):
+# kernel counts that are no multiple of 64 or 32 (padding lanes in the handed-over operand), a few-channel layer
+# in the middle (vector-ALU layer fed with fp32 by an fp4 layer, and feeding one), an fp4 layer first
+STACK2 = [
+    (TBN, (64, 12, 12, 70, 3, 3, 1, 1)),
+    (TNN, (70, 12, 12, 130, 3, 3, 1, 1)),
+    (BNN, (130, 12, 12, 16, 1, 1, 0, 1)),
+    (BTN, (16, 12, 12, 33, 3, 3, 1, 2)),
+    (TNN, (33, 6, 6, 200, 3, 3, 0, 1)),
+    (TBN, (200, 4, 4, 10, 4, 4, 0, 1)),
+]
+# larger pixel counts: the unsplit and the two-way split fp4 kernels, wide vector-ALU tiles in the stem
+STACK3 = [
+    (TNN, (3, 64, 64, 64, 7, 7, 3, 2)),
+    (TNN, (64, 32, 32, 64, 3, 3, 1, 1)),
+    (BTN, (64, 32, 32, 128, 3, 3, 1, 2)),
+    (TNN, (128, 16, 16, 32, 1, 1, 0, 1)),
+]
+
+
+def build(hip, oracle, batch, stack=None):
     import torch
     layers, host = [], []
-    for i, (typ, shape) in enumerate(STACK):
+    for i, (typ, shape) in enumerate(stack or STACK):
         c, ih, iw, kn, kw, kh, pad, stride = shape
         wt = weight_is_ternary(typ)
         w = synth.ternary(600 + i, (kn, c, kh, kw)) if wt else synth.binary(600 + i, (kn, c, kh, kw))
@@ -71,6 +90,28 @@ def test_chain_matches_the_oracle_layer_by_layer(hip, oracle):
         net.run(xd, out=out2, graph=True)
         s.synchronize()
         assert torch.equal(out, out2)
+    net.close()
+
+
+@pytest.mark.parametrize("which", [2, 3])
+def test_other_chains_match_the_oracle(hip, oracle, which):
+    import torch
+    stack, batch = (STACK2, 5) if which == 2 else (STACK3, 70)
+    net, host = build(hip, oracle, batch, stack)
+    c, ih, iw = stack[0][1][:3]
+    x = synth.normal(10 + which, (batch, c, ih, iw))
+    want = oracle_chain(oracle, host, x)
+    xd = torch.from_numpy(x).cuda()
+    got = net.run(xd)
+    assert got.cpu().numpy().tobytes() == want.tobytes()
+    s = torch.cuda.Stream()
+    out = torch.empty_like(got)
+    with torch.cuda.stream(s):
+        for rep in range(2):
+            out.fill_(-1.0)
+            net.run(xd, out=out, graph=True)
+            s.synchronize()
+            assert out.cpu().numpy().tobytes() == want.tobytes(), "replay %d" % rep
     net.close()
 
 

@@ -49,6 +49,9 @@ def test_layer_device_api(hip, oracle, typ, si, batch):
     _same_bits(y_d.cpu().numpy(), y_o, "GEMM output")
     yc_d = hip.conv(typ, x_d, thr_d, qw_d, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], L["alpha"])
     _same_bits(yc_d.cpu().numpy(), y_o, "conv output")
+    prepared = hip.prepare_conv_weights(typ, qw_d, L["c"], L["kn"], L["kh"], L["kw"])
+    yp_d = hip.conv_prepared(typ, x_d, thr_d, prepared, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], L["alpha"])
+    _same_bits(yp_d.cpu().numpy(), y_o, "conv output, prepared weights")
     for eng in (hip.ENGINE_VALU, hip.ENGINE_MFMA_F4):   # the layer on each engine explicitly
         ye_d = hip.conv(typ, x_d, thr_d, qw_d, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], L["alpha"],
                         engine=eng)
