@@ -298,11 +298,13 @@ struct ConvFrag {
 // (mm_p2_final_tnn_avx2.c:204-208), else "r >= 0 ? r : alpha * r" (mm_p2_final_tbn_avx2.c:73).
 // QMODE: 0 = fp32 NCHW result, 1 / 2 = ternary / binary hand-over to the next layer (QuantOut).
 // All three are compile-time so that the per-element epilogue carries no selects for them.
-template <bool ABIN, bool FORM0, int QMODE, int S>
-__global__ __launch_bounds__(256) void k_conv_f4(const uint4* __restrict__ P4, const uint4* __restrict__ Wf,
+// The unsplit hand-over variants are the ones launched with several thousand wavefronts (stems,
+// first stages): they are asked to fit three wavefronts per SIMD, which they do without scratch.
+template <bool ABIN, bool FORM0, int QMODE, int S, int NB>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && QMODE != 0) ? 3 : 1, 8))) void k_conv_f4(const uint4* __restrict__ P4, const uint4* __restrict__ Wf,
                                                  float* __restrict__ Y, int M, int KN, int OHW, int KB,
                                                  int bias, float alpha, FastDiv dOHW, ConvGeom cg, QuantOut qo) {
-    constexpr int NB = 3;                 // register sets of fragments: NB - 1 steps of loads in flight
+    // NB register sets of fragments: NB - 1 steps of loads in flight
     constexpr int PUB = 4 - 4 / S;        // blocks a wavefront hands to the others of its tile
     __shared__ float4 red[S > 1 ? 4 * PUB * 4 * 64 : 1];   // [wavefront][slot][e / 4][lane]
     const int tid = threadIdx.x, lane = tid & 63;
@@ -322,6 +324,14 @@ __global__ __launch_bounds__(256) void k_conv_f4(const uint4* __restrict__ P4, c
         ih0[b] = oh * cg.H_stride - cg.H_pad;
         iw0[b] = ow * cg.W_stride - cg.W_pad;
         pb[b] = n * (uint32_t)(cg.CP * cg.H * cg.W);   // image n of P4[n][C_pack][pixel]
+    }
+    // threshold of each pixel block's image for the hand-over, fetched now: behind the hand-counted loads
+    // below the compiler could only place this load where its value is used, at the very end
+    float qthr[2] = {0.0f, 0.0f};
+    if constexpr (QMODE != 0) {
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+            qthr[b] = qo.thr[fastdiv((uint32_t)min(px0 + 32 * b + lr, M - 1), dOHW)];
     }
     const int HWin = cg.H * cg.W;
     const int rbmax = (KN + 31) / 32 - 1;
@@ -486,7 +496,7 @@ __global__ __launch_bounds__(256) void k_conv_f4(const uint4* __restrict__ P4, c
                 // 8g + 4h + {0..3} of the block: half of nibble dword g of the pixel; the other
                 // half sits in lane ^ 32.  Lane h ends up with dwords 2h and 2h + 1 of the
                 // block's 16 bytes, i.e. bytes 16a + 8h .. + 8 of the pixel's 64-channel word.
-                const float t = qo.thr[img];
+                const float t = qthr[b];
                 constexpr bool tern = QMODE == 1;
                 const bool inside = kn0 + 32 * a + 32 <= KN;   // uniform: no per-kernel checks then
                 uint32_t half[4];
@@ -608,9 +618,10 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
     auto by_split = [&](auto abin, auto form0, auto qmode) -> hipError_t {
         constexpr bool A = decltype(abin)::value, F = decltype(form0)::value;
         constexpr int Q = decltype(qmode)::value;
-        if (split == 1) return launch(k_conv_f4<A, F, Q, 1>);
-        if (split == 2) return launch(k_conv_f4<A, F, Q, 2>);
-        if (split == 4) return launch(k_conv_f4<A, F, Q, 4>);
+        // three register sets: deeper prefetch measured no faster at any layer size
+        if (split == 1) return launch(k_conv_f4<A, F, Q, 1, 3>);
+        if (split == 2) return launch(k_conv_f4<A, F, Q, 2, 3>);
+        if (split == 4) return launch(k_conv_f4<A, F, Q, 4, 3>);
         return hipErrorInvalidValue;
     };
     auto by_mode = [&](auto abin, auto form0) -> hipError_t {
