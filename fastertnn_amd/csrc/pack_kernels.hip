@@ -326,63 +326,74 @@ __global__ __launch_bounds__(256) void k_quantize_nib(const float* __restrict__ 
     Pq[(size_t)n * HW + p] = dw;
 }
 
-// k_dense_rows_f4: one work-item per (output pixel, dense word d) strings the C nibbles of taps
-// d*T .. d*T + T - 1 together (lane (tap % T)*C + c, as in k_dense_rows), then the lanes left over,
-// 64 lanes = 32 bytes in all, and the block writes its 8 KiB through LDS in one contiguous piece.
-// Taps outside the image, taps past KH*KW and left-over lanes hold the padding lane of the type.
+// k_dense_rows_f4: one work-item per output pixel walks the KH*KW taps once and strings their C
+// nibbles together, T taps per 64-lane word (lane (tap % T)*C + c, as in k_dense_rows), closing each
+// word with the lanes left over: 64 lanes = 32 bytes per word.  A finished word goes through LDS so
+// that the block writes its 256 pixels x 32 bytes as one contiguous 8 KiB piece.  Taps outside the
+// image and left-over lanes hold the padding lane of the type.  The bit cursor depends on (C, T)
+// only, so it and every branch on it are wave-uniform.
 // Output = the fp4 layer kernel's operand for a 1x1 layer over the output pixels with Kd words per
 // pixel: A4[n][d][pixel][32 bytes].
 template <bool TERN>
 __global__ __launch_bounds__(256) void k_dense_rows_f4(const uint32_t* __restrict__ Pq, int C, int T, int H, int W,
                                                        int OHW, int OW, int KW, int taps, int Kd, int H_pad,
                                                        int W_pad, int H_stride, int W_stride, FastDiv dOW,
-                                                       FastDiv dKW, uint32_t* __restrict__ A4) {
+                                                       uint32_t* __restrict__ A4) {
     __shared__ uint32_t s_out[256 * 9];
-    const int pix = blockIdx.x * 256 + threadIdx.x, d = blockIdx.y, n = blockIdx.z;
+    const int pix0 = blockIdx.x * 256, n = blockIdx.y;
+    const int pix = min(pix0 + (int)threadIdx.x, OHW - 1);
     const uint32_t padv = TERN ? 0u : 0x22222222u;
-    if (pix < OHW) {
-        const int oh = (int)fastdiv((uint32_t)pix, dOW), ow = pix - oh * OW;
-        const int ih0 = oh * H_stride - H_pad, iw0 = ow * W_stride - W_pad;
-        const uint32_t* img = Pq + (size_t)n * H * W;
-        const uint32_t cmask = C >= 8 ? 0xffffffffu : ((1u << (4 * C)) - 1u);
-        const int tap0 = d * T;
-        int kh = (int)fastdiv((uint32_t)tap0, dKW), kw = tap0 - kh * KW;
+    const int oh = (int)fastdiv((uint32_t)pix, dOW), ow = pix - oh * OW;
+    const int ih0 = oh * H_stride - H_pad, iw0 = ow * W_stride - W_pad;
+    const uint32_t* img = Pq + (size_t)n * H * W;
+    const uint32_t cmask = C >= 8 ? 0xffffffffu : ((1u << (4 * C)) - 1u);
+    uint32_t* mine = s_out + threadIdx.x * 9;
+    int kh = 0, kw = 0, tap = 0;
+    for (int d = 0; d < Kd; d++) {
+        const int jn = min(T, taps - tap);   // taps of this word
         unsigned long long cur = 0ull;
         int pos = 0, k = 0;
-        uint32_t* mine = s_out + threadIdx.x * 9;
-        for (int j = 0; j <= T; j++) {
-            uint32_t v;
-            int bits;
-            if (j < T) {
+        for (int j0 = 0; j0 < jn; j0 += 8) {
+            // eight taps' loads in flight at once, then their nibbles are appended in order
+            uint32_t v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
                 const int ih = ih0 + kh, iw = iw0 + kw;
-                const bool in = tap0 + j < taps && (unsigned)ih < (unsigned)H && (unsigned)iw < (unsigned)W;
-                v = (in ? img[ih * W + iw] : padv) & cmask;
-                bits = 4 * C;
-                if (++kw == KW) {
+                const bool in = j0 + u < jn && (unsigned)ih < (unsigned)H && (unsigned)iw < (unsigned)W;
+                v[u] = in ? img[ih * W + iw] : padv;
+                if (j0 + u < jn && ++kw == KW) {
                     kw = 0;
                     kh++;
                 }
-            } else {   // the lanes left over after T taps
-                bits = 4 * (64 - T * C);
-                v = bits ? (padv & ((1u << bits) - 1u)) : 0u;   // bits < 32: fewer than C <= 8 lanes are left
             }
-            cur |= (unsigned long long)v << pos;
-            pos += bits;
-            if (pos >= 32) {
-                mine[k++] = (uint32_t)cur;
-                cur >>= 32;
-                pos -= 32;
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                if (j0 + u < jn) {   // uniform
+                    cur |= (unsigned long long)(v[u] & cmask) << pos;
+                    pos += 4 * C;
+                    if (pos >= 32) {
+                        mine[k++] = (uint32_t)cur;
+                        cur >>= 32;
+                        pos -= 32;
+                    }
+                }
             }
         }
-    }
-    __syncthreads();
-    // 256 pixels x 8 dwords, contiguous in A4 for this (n, d)
-    const int pix0 = blockIdx.x * 256;
-    uint32_t* dst = A4 + (((size_t)n * Kd + d) * OHW + pix0) * 8;
+        tap += jn;
+        // the lanes left over: 64 - jn*C of them, all padding
+        if (pos > 0) {
+            cur |= (unsigned long long)padv << pos;   // fills up to bit 32 + pos; bits past 32 are dropped below
+            mine[k++] = (uint32_t)cur;
+        }
+        for (; k < 8; k++) mine[k] = padv;
+        __syncthreads();
+        uint32_t* dst = A4 + (((size_t)n * Kd + d) * OHW + pix0) * 8;
 #pragma unroll
-    for (int it = 0; it < 8; it++) {
-        const int e = it * 256 + threadIdx.x;
-        if (pix0 + (e >> 3) < OHW) dst[e] = s_out[(e >> 3) * 9 + (e & 7)];
+        for (int it = 0; it < 8; it++) {
+            const int e = it * 256 + threadIdx.x;
+            if (pix0 + (e >> 3) < OHW) dst[e] = s_out[(e >> 3) * 9 + (e & 7)];
+        }
+        __syncthreads();
     }
 }
 
@@ -464,17 +475,15 @@ hipError_t launch_dense_rows_f4(bool ternary, const float* d_x, const float* d_t
     if (N > 65535 || Kd > 65535) return hipErrorInvalidValue;
     uint32_t* Pq = static_cast<uint32_t*>(d_pq);
     uint32_t* A4 = static_cast<uint32_t*>(d_a4);
-    dim3 gq((HW + 255) / 256, N), gr((OHW + 255) / 256, Kd, N);
+    dim3 gq((HW + 255) / 256, N), gr((OHW + 255) / 256, N);
     if (ternary) {
         hipLaunchKernelGGL((k_quantize_nib<true>), gq, dim3(256), 0, st, d_x, d_thr, C, HW, Pq);
         hipLaunchKernelGGL((k_dense_rows_f4<true>), gr, dim3(256), 0, st, Pq, C, T, H, W, OHW, OW, kW, kH * kW, Kd,
-                           H_pad, W_pad, H_stride, W_stride, make_fastdiv((uint32_t)OW), make_fastdiv((uint32_t)kW),
-                           A4);
+                           H_pad, W_pad, H_stride, W_stride, make_fastdiv((uint32_t)OW), A4);
     } else {
         hipLaunchKernelGGL((k_quantize_nib<false>), gq, dim3(256), 0, st, d_x, d_thr, C, HW, Pq);
         hipLaunchKernelGGL((k_dense_rows_f4<false>), gr, dim3(256), 0, st, Pq, C, T, H, W, OHW, OW, kW, kH * kW, Kd,
-                           H_pad, W_pad, H_stride, W_stride, make_fastdiv((uint32_t)OW), make_fastdiv((uint32_t)kW),
-                           A4);
+                           H_pad, W_pad, H_stride, W_stride, make_fastdiv((uint32_t)OW), A4);
     }
     return hipGetLastError();
 }
