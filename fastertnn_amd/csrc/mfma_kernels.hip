@@ -603,8 +603,9 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
     const FastDiv dOHW = make_fastdiv((uint32_t)OHW);
     // The kernel's hand-counted loads write registers behind the compiler's back; that is only
     // sound while none of its registers live in scratch memory, which is checked once per variant.
-    auto launch = [&](auto kern) -> hipError_t {
-        static const hipError_t sound = [&]() {
+    auto launch = [&](auto variant) -> hipError_t {   // variant: a distinct type per kernel instance
+        constexpr auto kern = decltype(variant)::value;
+        static const hipError_t sound = []() {      // hence one check per instance
             hipFuncAttributes attr;
             hipError_t e = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(kern));
             if (e == hipSuccess && attr.localSizeBytes != 0) e = hipErrorLaunchFailure;
@@ -619,9 +620,9 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
         constexpr bool A = decltype(abin)::value, F = decltype(form0)::value;
         constexpr int Q = decltype(qmode)::value;
         // three register sets: deeper prefetch measured no faster at any layer size
-        if (split == 1) return launch(k_conv_f4<A, F, Q, 1, 3>);
-        if (split == 2) return launch(k_conv_f4<A, F, Q, 2, 3>);
-        if (split == 4) return launch(k_conv_f4<A, F, Q, 4, 3>);
+        if (split == 1) return launch(std::integral_constant<decltype(&k_conv_f4<A, F, Q, 1, 3>), &k_conv_f4<A, F, Q, 1, 3>>{});
+        if (split == 2) return launch(std::integral_constant<decltype(&k_conv_f4<A, F, Q, 2, 3>), &k_conv_f4<A, F, Q, 2, 3>>{});
+        if (split == 4) return launch(std::integral_constant<decltype(&k_conv_f4<A, F, Q, 4, 3>), &k_conv_f4<A, F, Q, 4, 3>>{});
         return hipErrorInvalidValue;
     };
     auto by_mode = [&](auto abin, auto form0) -> hipError_t {

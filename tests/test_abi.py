@@ -137,3 +137,17 @@ def test_seeded_generators_are_pinned():
     g = synth.normal(1, (1 << 16,))
     assert abs(float(g.mean())) < 0.02 and abs(float(g.std()) - 1.0) < 0.02
     assert np.array_equal(synth.normal(9, (1000,))[100:200], synth.normal(9, (200,))[100:200])
+
+
+def test_build_refuses_scratch_in_hand_counted_kernels():
+    """the build's guard for kernels whose loads are counted by hand: scratch use there is an error"""
+    from fastertnn_amd import build
+    ok = ("x.hip:1:1: remark: Function Name: _ZN4ftnn9k_conv_f4ILb0EEEvv [-Rpass-analysis=kernel-resource-usage]\n"
+          "x.hip:1:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]\n"
+          "x.hip:1:1: remark: Function Name: _ZN4ftnn6k_mfmaEvv [-Rpass-analysis=kernel-resource-usage]\n"
+          "x.hip:1:1: remark:     ScratchSize [bytes/lane]: 64 [-Rpass-analysis=kernel-resource-usage]\n")
+    build.check_no_scratch("mfma_kernels.hip", ok)
+    with pytest.raises(RuntimeError, match="scratch"):
+        build.check_no_scratch("mfma_kernels.hip", ok.replace("lane]: 0", "lane]: 60"))
+    with pytest.raises(RuntimeError, match="no resource remarks"):
+        build.check_no_scratch("mfma_kernels.hip", "")
