@@ -164,6 +164,33 @@ def other_types(torch, lib, a_tern, b_tern, m, n, k, reps=5):
     return out
 
 
+def pack_rates(torch, lib, reps=10):
+    """the quantise + im2row + bit-pack stage alone (t2r_p2_opt / b2r on device memory): algorithmic bytes (fp32
+    input once, packed rows once) over the time of its two launches, against the 8 TB/s of HBM"""
+    out = {}
+    g = torch.Generator(device="cuda")
+    g.manual_seed(11)
+    for name, tern, (n, c, h, w, k, pad, stride) in (("t2r_b1_c256_56x56_k3", True, (1, 256, 56, 56, 3, 1, 1)),
+                                                      ("t2r_b32_c256_56x56_k3", True, (32, 256, 56, 56, 3, 1, 1)),
+                                                      ("b2r_b32_c256_56x56_k3", False, (32, 256, 56, 56, 3, 1, 1))):
+        x = torch.randn((n, c, h, w), generator=g, device="cuda")
+        thr = torch.full((n,), 0.5 if tern else 0.0, device="cuda")
+        oh, ow = lib.out_dim(h, pad, k, stride), lib.out_dim(w, pad, k, stride)
+        rows = torch.empty(n * oh * ow * lib.row_words(c, k, k, tern), dtype=torch.int64, device="cuda")
+        scratch = torch.empty(lib.pack_scratch_bytes(n, c, h, w, tern), dtype=torch.uint8, device="cuda")
+
+        def step():
+            lib.quantize_im2row(x, thr, k, k, pad, stride, tern, out=rows, scratch=scratch)
+        for _ in range(3):
+            step()
+        t = sorted(event_times(torch, step, reps))[reps // 2]
+        nbytes = 4.0 * x.numel() + 8.0 * rows.numel()
+        out[name] = {"ms": round(t, 4), "algorithmic_mb": round(nbytes / 1e6, 1), "gbps": round(nbytes / t / 1e6, 1),
+                     "frac_of_8tbps": round(nbytes / t / 1e6 / 8000.0, 3)}
+        del x, rows, scratch
+    return out
+
+
 def conv_latency(torch, lib, typ, shape, batch, seed, reps=20):
     """kernel-only (device buffers, HIP events) and ABI-inclusive (host pointers) latency"""
     import numpy as np
@@ -403,6 +430,7 @@ def main():
         extra = {
             "other_types_same_gemm_shape": other_types(torch, lib, a, b, m, n, k),
             "tnn_gemm_256x256x4096": small_gemm(torch, lib, 256, 256, 4096),
+            "quantize_im2row_pack": pack_rates(torch, lib),
             "tnn_conv_b1_c256_56x56_k3": conv_latency(torch, lib, TNN, (256, 56, 56, 256, 3, 3, 1, 1), 1, 2),
             "tbn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, TBN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 3),
             "btn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, BTN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 4),
