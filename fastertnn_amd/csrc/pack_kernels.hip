@@ -167,44 +167,47 @@ __global__ __launch_bounds__(256) void k_quantize_ballot(const float* __restrict
 }
 
 // ------------------------------------------------------------------ im2row
-// one work-item per output word (pair); lanes run along the row
+// One work-item per 16 bytes of output: two consecutive words of one plane of one group of 4 words of
+// one output row (ternary group = 4 sign words then 4 zero words, 64 bytes; binary group = 4 words, 32
+// bytes).  It gathers its two (tap, channel word) sources from P, or takes the fill
+// (src/tnns/ternarize2row_avx2.c:440-441,748-755; src/tnns/binarize2row_avx2.c:151).  Neighbouring
+// work-items write neighbouring 16 bytes, so every store instruction covers one contiguous KiB.
 template <bool TERN>
 __global__ __launch_bounds__(256) void k_im2row(const unsigned long long* __restrict__ P, int H,
-                                                int W, int CP, int OH, int OW, int KW, int K,
+                                                int W, int CP, int OHW, int OW, int KW, int K,
                                                 int Kw, int H_pad, int W_pad, int H_stride,
-                                                int W_stride, int64_t total,
-                                                unsigned long long* __restrict__ out) {
-    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+                                                int W_stride, int64_t total, FastDiv dPR, FastDiv dOHW,
+                                                FastDiv dOW, FastDiv dCP, FastDiv dKW,
+                                                ulonglong2* __restrict__ out) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;   // < 2^32, checked by the host
     if (e >= total) return;
-    const int64_t r = e / Kw;
-    const int idx = (int)(e - r * Kw);
-    unsigned long long s = 0ull, z = ~0ull;
-    if (idx < K) {
-        const int ic = idx % CP, tap = idx / CP;
-        const int kh = tap / KW, kw = tap - kh * KW;
-        const int ow = (int)(r % OW);
-        const int64_t t2 = r / OW;
-        const int oh = (int)(t2 % OH);
-        const int64_t n = t2 / OH;
-        const int ih = oh * H_stride + kh - H_pad, iw = ow * W_stride + kw - W_pad;
-        if (ih >= 0 && ih < H && iw >= 0 && iw < W) {
-            const size_t o = ((size_t)n * H * W + (size_t)ih * W + iw) * CP + ic;
-            if (TERN) {
-                const ulonglong2 v = reinterpret_cast<const ulonglong2*>(P)[o];
-                s = v.x;
-                z = v.y;
-            } else {
-                s = P[o];
+    constexpr int PPG = TERN ? 4 : 2;             // 16-byte pieces per group
+    const int PR = (Kw / 4) * PPG;                // pieces per row
+    const uint32_t r = fastdiv((uint32_t)e, dPR);
+    const int pr = (int)((uint32_t)e - r * (uint32_t)PR);
+    const int g = pr / PPG, piece = pr % PPG;
+    const bool zero_plane = TERN && piece >= 2;
+    const int idx0 = 4 * g + 2 * (piece & 1);     // first of the two words
+    const uint32_t n = fastdiv(r, dOHW), pix = r - n * (uint32_t)OHW;
+    const int oh = (int)fastdiv(pix, dOW), ow = (int)pix - oh * OW;
+    const int ih0 = oh * H_stride - H_pad, iw0 = ow * W_stride - W_pad;
+    const size_t img = (size_t)n * H * W;
+    unsigned long long v[2];
+#pragma unroll
+    for (int q = 0; q < 2; q++) {
+        const int idx = idx0 + q;
+        v[q] = zero_plane ? ~0ull : 0ull;
+        if (idx < K) {
+            const int tap = (int)fastdiv((uint32_t)idx, dCP), ic = idx - tap * CP;
+            const int kh = (int)fastdiv((uint32_t)tap, dKW), kw = tap - kh * KW;
+            const int ih = ih0 + kh, iw = iw0 + kw;
+            if ((unsigned)ih < (unsigned)H && (unsigned)iw < (unsigned)W) {
+                const size_t o = (img + (size_t)ih * W + iw) * CP + ic;
+                v[q] = TERN ? P[2 * o + (zero_plane ? 1 : 0)] : P[o];
             }
         }
     }
-    if (TERN) {
-        unsigned long long* row = out + (size_t)r * 2 * Kw;
-        row[p2_pos(idx, 0)] = s;
-        row[p2_pos(idx, 1)] = z;
-    } else {
-        out[(size_t)r * Kw + idx] = s;
-    }
+    out[e] = make_ulonglong2(v[0], v[1]);
 }
 
 // ------------------------------------------------------------- weight packers
@@ -550,15 +553,19 @@ hipError_t launch_quantize_im2row(bool ternary, const float* d_x, const float* d
     unsigned long long* P = static_cast<unsigned long long*>(d_scratch);
     hipError_t e = launch_quantize(ternary, d_x, d_thr, N, C, H, W, d_scratch, st);
     if (e != hipSuccess) return e;
-    const int64_t total = (int64_t)N * OH * OW * Kw;
+    const int pieces_per_row = (Kw / 4) * (ternary ? 4 : 2);   // 16-byte pieces
+    const int64_t total = (int64_t)N * OH * OW * pieces_per_row;
+    if (total > 0xffffffffLL) return hipErrorInvalidValue;
     const unsigned blocks = (unsigned)((total + 255) / 256);
-    unsigned long long* out = reinterpret_cast<unsigned long long*>(d_out);
+    ulonglong2* out = reinterpret_cast<ulonglong2*>(d_out);
+    const FastDiv dPR = make_fastdiv((uint32_t)pieces_per_row), dOHW = make_fastdiv((uint32_t)(OH * OW)),
+                  dOW = make_fastdiv((uint32_t)OW), dCP = make_fastdiv((uint32_t)CP), dKW = make_fastdiv((uint32_t)kW);
     if (ternary)
-        hipLaunchKernelGGL((k_im2row<true>), dim3(blocks), dim3(256), 0, st, P, H, W, CP, OH, OW, kW,
-                           K, Kw, H_pad, W_pad, H_stride, W_stride, total, out);
+        hipLaunchKernelGGL((k_im2row<true>), dim3(blocks), dim3(256), 0, st, P, H, W, CP, OH * OW, OW, kW,
+                           K, Kw, H_pad, W_pad, H_stride, W_stride, total, dPR, dOHW, dOW, dCP, dKW, out);
     else
-        hipLaunchKernelGGL((k_im2row<false>), dim3(blocks), dim3(256), 0, st, P, H, W, CP, OH, OW,
-                           kW, K, Kw, H_pad, W_pad, H_stride, W_stride, total, out);
+        hipLaunchKernelGGL((k_im2row<false>), dim3(blocks), dim3(256), 0, st, P, H, W, CP, OH * OW, OW,
+                           kW, K, Kw, H_pad, W_pad, H_stride, W_stride, total, dPR, dOHW, dOW, dCP, dKW, out);
     return hipGetLastError();
 }
 
