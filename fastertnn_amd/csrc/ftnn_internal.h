@@ -49,8 +49,17 @@ struct QuantOut {
 // the E2M1 nibble of one value under QuantOut mode 1 / 2 (src/tnns/ternarize2row_avx2.c:443-449,
 // src/tnns/binarize2row_avx2.c:19-21); `live` = false gives the padding lane of that mode
 __device__ __forceinline__ uint32_t quant_nibble(float v, float t, bool ternary, bool live) {
-    if (ternary) return live ? (v < -t ? 0xAu : (v > t ? 0x2u : 0x0u)) : 0x0u;
-    return live ? (v < t ? 0xAu : 0x2u) : 0x2u;
+    // selects only: a branch per element costs more than the whole computation
+    uint32_t r;
+    if (ternary) {
+        r = v > t ? 0x2u : 0x0u;
+        r = v < -t ? 0xAu : r;
+        r = live ? r : 0x0u;
+    } else {
+        r = v < t ? 0xAu : 0x2u;
+        r = live ? r : 0x2u;
+    }
+    return r;
 }
 
 // record a failure text for ftnn_last_error(); returns `code`

@@ -498,15 +498,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
                 // block's 16 bytes, i.e. bytes 16a + 8h .. + 8 of the pixel's 64-channel word.
                 const float t = qthr[b];
                 constexpr bool tern = QMODE == 1;
-                const bool inside = kn0 + 32 * a + 32 <= KN;   // uniform: no per-kernel checks then
                 uint32_t half[4];
+                if (kn0 + 32 * a + 32 <= KN) {   // uniform: the whole block holds real kernels
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    half[g] = 0u;
+                    for (int g = 0; g < 4; g++) {
+                        half[g] = 0u;
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const bool live = inside || kn0 + 32 * a + 8 * g + 4 * h + i < KN;
-                        half[g] |= quant_nibble(vals[4 * g + i], t, tern, live) << (4 * i);
+                        for (int i = 0; i < 4; i++) half[g] |= quant_nibble(vals[4 * g + i], t, tern, true) << (4 * i);
+                    }
+                } else {
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        half[g] = 0u;
+#pragma unroll
+                        for (int i = 0; i < 4; i++)
+                            half[g] |= quant_nibble(vals[4 * g + i], t, tern, kn0 + 32 * a + 8 * g + 4 * h + i < KN)
+                                       << (4 * i);
                     }
                 }
                 const uint32_t send = h ? (half[0] | (half[1] << 16)) : (half[2] | (half[3] << 16));

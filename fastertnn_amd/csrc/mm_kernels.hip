@@ -324,9 +324,14 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
                 const uint32_t pix = (uint32_t)i - img * (uint32_t)OHW;
                 const float t = qo.thr[img];
                 uint32_t dw = 0u;
+                const bool tern = qo.mode == 1;
+                if (col0 + TN <= KN) {   // uniform: all of this wavefront's columns are real kernels
 #pragma unroll
-                for (int b = 0; b < TN; b++)
-                    dw |= quant_nibble(finish(a, b), t, qo.mode == 1, col0 + b < KN) << (4 * b);
+                    for (int b = 0; b < TN; b++) dw |= quant_nibble(finish(a, b), t, tern, true) << (4 * b);
+                } else {
+#pragma unroll
+                    for (int b = 0; b < TN; b++) dw |= quant_nibble(finish(a, b), t, tern, col0 + b < KN) << (4 * b);
+                }
                 const size_t word = ((size_t)img * ((KN + 63) / 64) + (col0 >> 6)) * OHW + pix;
                 unsigned char* dst = static_cast<unsigned char*>(qo.p4) + word * 32 + ((col0 & 63) >> 1);
                 if (TN == 8) *reinterpret_cast<uint32_t*>(dst) = dw;
