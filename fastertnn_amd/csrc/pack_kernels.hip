@@ -330,73 +330,55 @@ __global__ __launch_bounds__(256) void k_quantize_nib(const float* __restrict__ 
 }
 
 // k_dense_rows_f4: one work-item per output pixel walks the KH*KW taps once and strings their C
-// nibbles together, T taps per 64-lane word (lane (tap % T)*C + c, as in k_dense_rows), closing each
-// word with the lanes left over: 64 lanes = 32 bytes per word.  A finished word goes through LDS so
-// that the block writes its 256 pixels x 32 bytes as one contiguous 8 KiB piece.  Taps outside the
-// image and left-over lanes hold the padding lane of the type.  The bit cursor depends on (C, T)
-// only, so it and every branch on it are wave-uniform.
+// nibbles together, T = 64 / C taps per 64-lane word (lane (tap % T)*C + c, as in k_dense_rows), the
+// lanes left over holding the padding lane of the type like taps outside the image.  C is a template
+// parameter: every shift and every position in the word's eight dwords is then a constant, the word
+// is assembled in registers and leaves as two 16-byte stores (32 contiguous bytes per pixel,
+// neighbouring pixels next to each other).
 // Output = the fp4 layer kernel's operand for a 1x1 layer over the output pixels with Kd words per
 // pixel: A4[n][d][pixel][32 bytes].
-template <bool TERN>
-__global__ __launch_bounds__(256) void k_dense_rows_f4(const uint32_t* __restrict__ Pq, int C, int T, int H, int W,
-                                                       int OHW, int OW, int KW, int taps, int Kd, int H_pad,
-                                                       int W_pad, int H_stride, int W_stride, FastDiv dOW,
-                                                       uint32_t* __restrict__ A4) {
-    __shared__ uint32_t s_out[256 * 9];
-    const int pix0 = blockIdx.x * 256, n = blockIdx.y;
-    const int pix = min(pix0 + (int)threadIdx.x, OHW - 1);
-    const uint32_t padv = TERN ? 0u : 0x22222222u;
+template <bool TERN, int C>
+__global__ __launch_bounds__(256) void k_dense_rows_f4(const uint32_t* __restrict__ Pq, int H, int W, int OHW,
+                                                       int OW, int KW, int taps, int Kd, int H_pad, int W_pad,
+                                                       int H_stride, int W_stride, FastDiv dOW,
+                                                       uint4* __restrict__ A4) {
+    constexpr int T = 64 / C;
+    constexpr uint32_t padv = TERN ? 0u : 0x22222222u;
+    constexpr uint32_t cmask = C >= 8 ? 0xffffffffu : ((1u << (4 * (C & 7))) - 1u);
+    const int pix = blockIdx.x * 256 + threadIdx.x, n = blockIdx.y;
+    if (pix >= OHW) return;
     const int oh = (int)fastdiv((uint32_t)pix, dOW), ow = pix - oh * OW;
     const int ih0 = oh * H_stride - H_pad, iw0 = ow * W_stride - W_pad;
     const uint32_t* img = Pq + (size_t)n * H * W;
-    const uint32_t cmask = C >= 8 ? 0xffffffffu : ((1u << (4 * C)) - 1u);
-    uint32_t* mine = s_out + threadIdx.x * 9;
     int kh = 0, kw = 0, tap = 0;
     for (int d = 0; d < Kd; d++) {
-        const int jn = min(T, taps - tap);   // taps of this word
-        unsigned long long cur = 0ull;
-        int pos = 0, k = 0;
-        for (int j0 = 0; j0 < jn; j0 += 8) {
-            // eight taps' loads in flight at once, then their nibbles are appended in order
-            uint32_t v[8];
+        uint32_t o[8];
 #pragma unroll
-            for (int u = 0; u < 8; u++) {
-                const int ih = ih0 + kh, iw = iw0 + kw;
-                const bool in = j0 + u < jn && (unsigned)ih < (unsigned)H && (unsigned)iw < (unsigned)W;
-                v[u] = in ? img[ih * W + iw] : padv;
-                if (j0 + u < jn && ++kw == KW) {
-                    kw = 0;
-                    kh++;
-                }
+        for (int i = 0; i < 8; i++) o[i] = padv;   // left-over lanes and missing taps stay padding
+#pragma unroll
+        for (int j = 0; j < T; j++) {
+            const int ih = ih0 + kh, iw = iw0 + kw;
+            const bool in = tap < taps && (unsigned)ih < (unsigned)H && (unsigned)iw < (unsigned)W;
+            // the load is unconditional (pixel 0 stands in for a tap outside the image) so that all T loads
+            // of a word can be in flight together
+            const uint32_t raw = img[in ? ih * W + iw : 0];
+            const uint32_t v = (in ? raw : padv) & cmask;
+            if (++kw == KW) {
+                kw = 0;
+                kh++;
             }
-#pragma unroll
-            for (int u = 0; u < 8; u++) {
-                if (j0 + u < jn) {   // uniform
-                    cur |= (unsigned long long)(v[u] & cmask) << pos;
-                    pos += 4 * C;
-                    if (pos >= 32) {
-                        mine[k++] = (uint32_t)cur;
-                        cur >>= 32;
-                        pos -= 32;
-                    }
-                }
+            tap++;
+            // lanes [j*C, j*C + C) of the word: bits [4*j*C, 4*j*C + 4*C) of its eight dwords
+            const int bit = 4 * j * C, lo = bit >> 5, sh = bit & 31;
+            o[lo] = (o[lo] & ~(cmask << sh)) | (v << sh);
+            if (sh + 4 * C > 32) {   // compile-time after unrolling: the tap straddles two dwords
+                const int rest = 32 - sh;
+                o[lo + 1] = (o[lo + 1] & ~(cmask >> rest)) | (v >> rest);
             }
         }
-        tap += jn;
-        // the lanes left over: 64 - jn*C of them, all padding
-        if (pos > 0) {
-            cur |= (unsigned long long)padv << pos;   // fills up to bit 32 + pos; bits past 32 are dropped below
-            mine[k++] = (uint32_t)cur;
-        }
-        for (; k < 8; k++) mine[k] = padv;
-        __syncthreads();
-        uint32_t* dst = A4 + (((size_t)n * Kd + d) * OHW + pix0) * 8;
-#pragma unroll
-        for (int it = 0; it < 8; it++) {
-            const int e = it * 256 + threadIdx.x;
-            if (pix0 + (e >> 3) < OHW) dst[e] = s_out[(e >> 3) * 9 + (e & 7)];
-        }
-        __syncthreads();
+        uint4* dst = A4 + (((size_t)n * Kd + d) * OHW + pix) * 2;
+        dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
+        dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
     }
 }
 
@@ -477,17 +459,26 @@ hipError_t launch_dense_rows_f4(bool ternary, const float* d_x, const float* d_t
     const int HW = H * W, OHW = OH * OW;
     if (N > 65535 || Kd > 65535) return hipErrorInvalidValue;
     uint32_t* Pq = static_cast<uint32_t*>(d_pq);
-    uint32_t* A4 = static_cast<uint32_t*>(d_a4);
+    uint4* A4 = static_cast<uint4*>(d_a4);
     dim3 gq((HW + 255) / 256, N), gr((OHW + 255) / 256, N);
-    if (ternary) {
-        hipLaunchKernelGGL((k_quantize_nib<true>), gq, dim3(256), 0, st, d_x, d_thr, C, HW, Pq);
-        hipLaunchKernelGGL((k_dense_rows_f4<true>), gr, dim3(256), 0, st, Pq, C, T, H, W, OHW, OW, kW, kH * kW, Kd,
-                           H_pad, W_pad, H_stride, W_stride, make_fastdiv((uint32_t)OW), A4);
-    } else {
-        hipLaunchKernelGGL((k_quantize_nib<false>), gq, dim3(256), 0, st, d_x, d_thr, C, HW, Pq);
-        hipLaunchKernelGGL((k_dense_rows_f4<false>), gr, dim3(256), 0, st, Pq, C, T, H, W, OHW, OW, kW, kH * kW, Kd,
-                           H_pad, W_pad, H_stride, W_stride, make_fastdiv((uint32_t)OW), A4);
+    const FastDiv dOW = make_fastdiv((uint32_t)OW);
+    (void)T;
+    if (ternary) hipLaunchKernelGGL((k_quantize_nib<true>), gq, dim3(256), 0, st, d_x, d_thr, C, HW, Pq);
+    else hipLaunchKernelGGL((k_quantize_nib<false>), gq, dim3(256), 0, st, d_x, d_thr, C, HW, Pq);
+#define FTNN_DENSE(C_)                                                                                              \
+    case C_:                                                                                                        \
+        if (ternary)                                                                                                \
+            hipLaunchKernelGGL((k_dense_rows_f4<true, C_>), gr, dim3(256), 0, st, Pq, H, W, OHW, OW, kW, kH * kW, Kd,  \
+                               H_pad, W_pad, H_stride, W_stride, dOW, A4);                                          \
+        else                                                                                                        \
+            hipLaunchKernelGGL((k_dense_rows_f4<false, C_>), gr, dim3(256), 0, st, Pq, H, W, OHW, OW, kW, kH * kW, Kd, \
+                               H_pad, W_pad, H_stride, W_stride, dOW, A4);                                          \
+        break;
+    switch (C) {
+        FTNN_DENSE(1) FTNN_DENSE(2) FTNN_DENSE(3) FTNN_DENSE(4) FTNN_DENSE(5) FTNN_DENSE(6) FTNN_DENSE(7) FTNN_DENSE(8)
+        default: return hipErrorInvalidValue;
     }
+#undef FTNN_DENSE
     return hipGetLastError();
 }
 
