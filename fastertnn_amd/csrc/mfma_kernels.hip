@@ -278,8 +278,8 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
 //   * a wavefront owns 64 kernels x 64 output pixels (2 x 2 MFMA blocks, 64 accumulator
 //     registers).  A workgroup is 4 wavefronts: S of them split the K loop of one tile (word w of
 //     the reference's K order (kh*KW + kw)*C_pack + ic goes to wavefront w % S of the tile), so
-//     it covers 4/S pixel tiles.  S = 1 for layers with many pixels (no exchange at all), 2 or 4
-//     where the tiles alone would leave most of the chip idle; the partial tiles then meet in
+//     it covers 4/S pixel tiles.  S = 1 for layers with 600 tiles or more (no exchange at all), 2 or
+//     4 where the tiles alone would leave most of the chip idle; the partial tiles then meet in
 //     LDS and each wavefront finishes 4/S of the tile's four blocks;
 //   * weights are the MFMA A side (rows = accumulator registers), pixels the B side (rows =
 //     lanes), so a store instruction writes 32 consecutive pixels of one NCHW plane;
@@ -305,13 +305,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
                                                  float* __restrict__ Y, int M, int KN, int OHW, int KB,
                                                  int bias, float alpha, FastDiv dOHW, ConvGeom cg, QuantOut qo) {
     // NB register sets of fragments: NB - 1 steps of loads in flight
+    constexpr int WPB = 4;                // wavefronts per workgroup (single-wavefront workgroups for S = 1
+                                          // measured slower: neighbours no longer share weight fragments in L1)
     constexpr int PUB = 4 - 4 / S;        // blocks a wavefront hands to the others of its tile
     __shared__ float4 red[S > 1 ? 4 * PUB * 4 * 64 : 1];   // [wavefront][slot][e / 4][lane]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ks = wave % S, pt = wave / S;   // K share and pixel tile of this wavefront
     const int h = lane >> 5, lr = lane & 31;
-    const int px0 = (blockIdx.x * (4 / S) + pt) * 64, kn0 = blockIdx.y * 64;
+    const int px0 = (blockIdx.x * (WPB / S) + pt) * 64, kn0 = blockIdx.y * 64;
 
     int ih0[2], iw0[2];
     uint32_t pb[2];
@@ -600,10 +602,11 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
     // K split: enough wavefronts to occupy the chip's 1024 SIMDs, but no exchange where the tiles
     // alone do that (a tile = 64 kernels x 64 pixels)
     const int64_t tiles = ((M + 63) / 64) * ((KN + 63) / 64);
-    int split = tiles >= 1024 ? 1 : (tiles >= 512 ? 2 : 4);
+    int split = tiles >= 600 ? 1 : (tiles >= 450 ? 2 : 4);   // measured on MI355X (1024 SIMDs)
     static const char* tune = getenv("FTNN_CONV_SPLIT");   // tuning aid: force the K split
     if (tune) split = atoi(tune);
-    dim3 grid((unsigned)(((M + 63) / 64 + 4 / split - 1) / (4 / split)), (unsigned)((KN + 63) / 64));
+    const int wpb = 4, tpb = wpb / split;   // wavefronts and pixel tiles per workgroup (see the kernel)
+    dim3 grid((unsigned)(((M + 63) / 64 + tpb - 1) / tpb), (unsigned)((KN + 63) / 64));
     if (M > 0x7fffff00LL || grid.y > 65535) return hipErrorInvalidValue;   // pixel indices stay below 2^31
     const uint4* P4 = static_cast<const uint4*>(d_p4);
     const uint4* Wf = static_cast<const uint4*>(d_wf);
@@ -619,7 +622,7 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
             return e;
         }();
         if (sound != hipSuccess) return sound;
-        hipLaunchKernelGGL(kern, grid, dim3(256), 0, st, P4, Wf, d_y, (int)M, KN, OHW, KB, bias, alpha, dOHW, cg, qo);
+        hipLaunchKernelGGL(kern, grid, dim3(64 * wpb), 0, st, P4, Wf, d_y, (int)M, KN, OHW, KB, bias, alpha, dOHW, cg, qo);
         return hipGetLastError();
     };
     // kernel variant: activation kind and PReLU form follow the type, then hand-over mode and split
