@@ -107,3 +107,28 @@ def test_engine_argument_checks(hip):
     assert hip.mm_scratch_bytes(hip.ENGINE_MFMA_I8, 0, 33, 1, 1, 1, 4) == (2 + 1) * 8 * 1024
     assert hip.select_engine(0, 8192, 1, 1, 8192, 512) == hip.ENGINE_MFMA_F4
     assert hip.select_engine(0, 1, 56, 56, 256, 36) == hip.ENGINE_VALU
+
+
+def test_layer_engine_argument_checks(hip):
+    import torch
+    x = torch.zeros((2, 64, 8, 8), device="cuda")
+    thr = torch.zeros(2, device="cuda")
+    qw = torch.zeros(16 * 2 * 12, dtype=torch.int64, device="cuda")
+    scratch = torch.empty(hip.conv_scratch_bytes(0, 2, 64, 8, 8, 16, 3, 3, 1, 1), dtype=torch.uint8, device="cuda")
+    y = torch.empty((2, 16, 8, 8), device="cuda")
+    L, s = hip._L, hip._stream()
+    args = (0, x.data_ptr(), thr.data_ptr(), qw.data_ptr(), 2, 64, 8, 8, 16, 3, 3, 1, 1, 1, 1, 0.5, scratch.data_ptr(),
+            y.data_ptr(), s)
+    assert L.ftnn_conv_engine(hip.ENGINE_MFMA_I8, *args) == -1          # layers run on the vector ALU or on fp4
+    assert b"engine" in L.ftnn_last_error()
+    assert L.ftnn_conv_engine(7, *args) == -1
+    for eng in (hip.ENGINE_AUTO, hip.ENGINE_VALU, hip.ENGINE_MFMA_F4):
+        assert L.ftnn_conv_engine(eng, *args) == 0
+    bad = list(args)
+    bad[16] = scratch.data_ptr() + 4                                     # misaligned scratch
+    assert L.ftnn_conv_engine(hip.ENGINE_MFMA_F4, *bad) == -1
+    assert L.ftnn_conv_prepared(0, x.data_ptr(), thr.data_ptr(), None, 2, 64, 8, 8, 16, 3, 3, 1, 1, 1, 1, 0.5,
+                                scratch.data_ptr(), y.data_ptr(), s) == -1
+    assert L.ftnn_conv_weights_bytes(0, 64, 16, 3, 3) == 1 * 12 * 1024    # one block of 32 kernels x 12 words
+    assert L.ftnn_conv_weights_bytes(5, 64, 16, 3, 3) == 0
+    torch.cuda.synchronize()
