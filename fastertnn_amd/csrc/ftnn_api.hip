@@ -463,14 +463,16 @@ int ftnn_conv_engine(int engine, int type, const float* d_x, const float* d_thr,
     if (!aligned16(d_scratch) || !aligned16(d_qw))
         return fail(FTNN_EINVAL, "d_scratch and d_qw must be 16-byte aligned");
     if ((int64_t)N * OH * OW > 0x7fffffffLL) return fail(FTNN_EINVAL, "more than 2^31-1 output rows");
-    if (engine == FTNN_ENGINE_AUTO) engine = select_conv_engine(type, N, C, H, W, KN, KH, KW, OH, OW);
+    const bool fits_f4 = (int64_t)N * H * W * cpack_of(C) <= 0x7fffffffLL &&
+                         (int64_t)N * OH * OW * conv_f4_weight_words(C, KH, KW) <= 0x7fffffffLL;
+    if (engine == FTNN_ENGINE_AUTO)   // a layer beyond the fp4 kernel's 32-bit pixel indices goes to the vector ALU
+        engine = fits_f4 ? select_conv_engine(type, N, C, H, W, KN, KH, KW, OH, OW) : FTNN_ENGINE_VALU;
     const bool w_ternary = (type == kTNN || type == kBTN);
     if (engine == FTNN_ENGINE_MFMA_F4) {
         const int Kw = conv_f4_weight_words(C, KH, KW);
         if (64LL * Kw >= (1LL << 24))
             return fail(FTNN_EINVAL, "K too long for exact fp32 accumulation; use the vector-ALU engine");
-        if ((int64_t)N * H * W * cpack_of(C) > 0x7fffffffLL || (int64_t)N * OH * OW * Kw > 0x7fffffffLL)
-            return fail(FTNN_EINVAL, "more than 2^31-1 input pixel words");
+        if (!fits_f4) return fail(FTNN_EINVAL, "more than 2^31-1 input pixel words: use the vector-ALU engine");
         char* d_wf = static_cast<char*>(d_scratch) + conv_f4_operand_bytes(N, C, H, W, KH, KW, OH, OW);
         const int64_t* rows = d_qw;
         hipError_t e;

@@ -118,6 +118,9 @@ ftnn_net_t* ftnn_net_create(int batch, int n_layers, const ftnn_layer_t* layers)
         const ftnn_layer_t& L = layers[i];
         f4[i] = ftnn_select_conv_engine(L.type, batch, L.C, L.H, L.W, L.KN, L.KH, L.KW, L.pad, L.pad, L.stride,
                                         L.stride) == FTNN_ENGINE_MFMA_F4;
+        if (f4[i] && ((int64_t)batch * L.H * L.W * cpack_of(L.C) > 0x7fffffffLL ||
+                      (int64_t)batch * net->OH[i] * net->OW[i] * conv_f4_weight_words(L.C, L.KH, L.KW) > 0x7fffffffLL))
+            f4[i] = 0;   // beyond the 32-bit pixel indices of the fp4 layer kernel: the vector-ALU layer takes it
         if (f4[i]) {
             max_p4 = std::max(max_p4, conv_f4_operand_bytes(batch, L.C, L.H, L.W, L.KH, L.KW, net->OH[i], net->OW[i]));
             if (i > 0 && dense_f4_applies(L.C, L.KH, L.KW))   // its input arrives as fp32
