@@ -238,9 +238,13 @@ FTNN_API int ftnn_conv_prepared(int type, const float *d_x, const float *d_thr, 
 /*
  * A chain of conv layers with device-resident activations: the e2e mode of the reference's
  * layer driver (src/timing_layers.c:182-207 feeds each layer's output to the next one), here
- * without the host round trip per layer.  All device memory (two activation buffers, the
- * quantiser scratch, per-layer threshold arrays) is allocated by ftnn_net_create; a run
- * allocates nothing.  Packed weights stay the caller's and must outlive the net.
+ * without the host round trip per layer.  A layer that feeds a layer on the fp4 matrix-core
+ * engine thresholds its own results with that layer's threshold and writes its quantised
+ * input directly, so no fp32 tensor exists between them; the chain's output is what the
+ * reference's chain of tnns_conv calls returns, bit for bit.  All device memory (activation
+ * and operand buffers, work space, per-layer threshold arrays, the weights in engine form) is
+ * allocated by ftnn_net_create; a run allocates nothing.  Packed weights stay the caller's and
+ * must outlive the net.
  */
 typedef struct ftnn_layer {
     int type;             /* TNN / TBN / BTN / BNN                               */
