@@ -271,9 +271,9 @@ RESNET18_LIKE = [  # (C, IH, IW, KN, KW, KH, pad, stride): stem, four stages wit
 ]
 
 
-def e2e_latency(torch, lib, batch, reps=10):
-    """the batch-32 ResNet-18-like TNN stack chained on the device (eager launches and HIP-graph
-    replay), and the same chain through the reference's tnns_conv on one host core"""
+def e2e_latency(torch, lib, batch, reps=10, cpu=True):
+    """the ResNet-18-like TNN stack chained on the device (eager launches and HIP-graph replay), and
+    (cpu=True) the same chain through the reference's tnns_conv on one host core"""
     import numpy as np
     from fastertnn_amd import TNN
     g = torch.Generator(device="cuda")
@@ -298,7 +298,7 @@ def e2e_latency(torch, lib, batch, reps=10):
             out[key] = round(t, 4)
     st.synchronize()
     from oracle import ftnn_oracle as O
-    if O.Reference.available():
+    if cpu and O.Reference.available():
         ref = O.Reference()
         xh = x.cpu().numpy()
         thr = np.full(batch, 0.5, np.float32)
@@ -435,6 +435,7 @@ def main():
             "tbn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, TBN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 3),
             "btn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, BTN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 4),
             "tnn_resnet18_like_b32_e2e": e2e_latency(torch, lib, 32),
+            "tnn_resnet18_like_other_batches": {"b%d" % b: e2e_latency(torch, lib, b, cpu=False) for b in (1, 8, 128)},
         }
 
     line = {
