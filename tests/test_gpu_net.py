@@ -4,7 +4,7 @@ replays are checked one by one against the eager result with other work in betwe
 import numpy as np
 import pytest
 
-from fastertnn_amd import synth, TNN, TBN, BTN, BNN, act_is_ternary, weight_is_ternary
+from fastertnn_amd import synth, TNN, TBN, BTN, BNN, TYPE_NAMES, act_is_ternary, weight_is_ternary
 
 pytestmark = pytest.mark.gpu
 
@@ -122,3 +122,46 @@ def test_chain_rejects_mismatched_layers(hip, oracle):
     bad = dict(type=TNN, shape=(32, 8, 8, 64, 1, 1, 0, 1), threshold=0.5, alpha=0.5, qw=qw)
     with pytest.raises(hip.FtnnError, match="not the output"):
         hip.Net(2, [good, bad])
+
+
+def test_random_chains_match_the_oracle(hip, oracle):
+    """seeded random chains of 2-5 layers: every type, thresholds and PReLU slopes of either sign, kernel
+    counts around the 32- and 64-channel word boundaries, few-channel inputs -- the quantised hand-over between
+    layers must not change a single output bit"""
+    import torch
+    rng = np.random.default_rng(2024)
+    done = 0
+    while done < 150:
+        batch = int(rng.integers(1, 7))
+        c = int(rng.choice([1, 3, 4, 8, 12, 32, 64, 70, 128, 192]))
+        h, w = int(rng.integers(4, 30)), int(rng.integers(4, 30))
+        x = synth.normal(int(rng.integers(1, 1 << 30)), (batch, c, h, w))
+        layers, host = [], []
+        for _ in range(int(rng.integers(2, 6))):
+            typ = int(rng.integers(0, 4))
+            kh, kw = int(rng.integers(1, 5)), int(rng.integers(1, 5))
+            pad, stride = int(rng.integers(0, 3)), int(rng.integers(1, 3))
+            if h + 2 * pad < kh or w + 2 * pad < kw:
+                break
+            kn = int(rng.choice([1, 5, 16, 33, 64, 65, 100, 128, 130, 200]))
+            wt = weight_is_ternary(typ)
+            seed = int(rng.integers(1, 1 << 30))
+            wgt = synth.ternary(seed, (kn, c, kh, kw)) if wt else synth.binary(seed, (kn, c, kh, kw))
+            qw = oracle.pack_weights(wgt, np.full(kn, 0.5 if wt else 0.0, np.float32), wt)
+            thr = float(rng.choice([0.5, 0.0, 1.5, 3.0])) if act_is_ternary(typ) else float(rng.choice([0.0, 0.5, -1.0]))
+            alpha = float(rng.choice([0.5, 0.25, 1.0, 0.0, -0.5]))
+            host.append((typ, (c, h, w, kn, kw, kh, pad, stride), qw, thr, alpha))
+            layers.append(dict(type=typ, shape=(c, h, w, kn, kw, kh, pad, stride), threshold=thr, alpha=alpha,
+                               qw=torch.from_numpy(qw).cuda()))
+            c, h, w = kn, (h + 2 * pad - kh) // stride + 1, (w + 2 * pad - kw) // stride + 1
+        if len(layers) < 2:
+            continue
+        print("chain", done, [(TYPE_NAMES[t], s) for t, s, _, _, _ in host], "batch", batch, flush=True)
+        want = x
+        for typ, (_, _, _, kn, kw, kh, pad, stride), qw, thr, alpha in host:
+            want = oracle.conv(typ, want, np.full(want.shape[0], thr, np.float32), qw, kn, kh, kw, pad, stride, alpha)
+        net = hip.Net(batch, layers)
+        got = net.run(torch.from_numpy(x).cuda()).cpu().numpy()
+        net.close()
+        assert got.tobytes() == np.ascontiguousarray(want).tobytes()
+        done += 1
