@@ -312,6 +312,57 @@ def e2e_latency(torch, lib, batch, reps=10, cpu=True):
     return out
 
 
+def reference_networks(torch, lib, batch=8, reps=5):
+    """the networks of the reference's e2e mode that chain shape to shape (include/timing/shapes_e2e.h, kept as
+    data in tests/golden/reference_shape_tables.json), at the reference's batch of 8 (src/timing_layers.c:46):
+    device-resident layer chain against the same tnns_conv chain on one host core"""
+    import numpy as np
+    from fastertnn_amd import TNN
+    from oracle import ftnn_oracle as O
+    tables = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "golden",
+                                         "reference_shape_tables.json")))
+    out = {}
+    g = torch.Generator(device="cuda")
+    g.manual_seed(8)
+    for net_t in tables["e2e"]:
+        shapes = [tuple(r) for r in net_t["layers"]]
+        c, h, w = shapes[0][:3]
+        ok = True
+        for (cc, ih, iw, kn, kw, kh, p, s) in shapes:
+            ok = ok and (cc, ih, iw) == (c, h, w)
+            c, h, w = kn, lib.out_dim(ih, p, kh, s), lib.out_dim(iw, p, kw, s)
+        if not ok:
+            continue   # the table leaves out pooling layers: not a chain
+        layers = []
+        for (c, ih, iw, kn, kw, kh, p, s) in shapes:
+            wgt = torch.randint(-1, 2, (kn, c, kh, kw), generator=g, device="cuda", dtype=torch.int8).float()
+            qw = lib.pack_weights(wgt, torch.full((kn,), 0.5, device="cuda"), True)
+            layers.append(dict(type=TNN, shape=(c, ih, iw, kn, kw, kh, p, s), threshold=0.5, alpha=0.5, qw=qw))
+        x = torch.randn((batch,) + shapes[0][:3], generator=g, device="cuda")
+        net = lib.Net(batch, layers)
+        y = torch.empty(net.out_shape, device="cuda")
+        for _ in range(2):
+            net.run(x, out=y)
+        t = sorted(event_times(torch, lambda: net.run(x, out=y), reps))[reps // 2]
+        macs = sum(batch * lib.out_dim(ih, p, kh, s) * lib.out_dim(iw, p, kw, s) * kn * c * kh * kw
+                   for (c, ih, iw, kn, kw, kh, p, s) in shapes)
+        row = {"layers": len(shapes), "gmac": round(macs / 1e9, 1), "device_ms": round(t, 4)}
+        if O.Reference.available():
+            ref = O.Reference()
+            xh = x.cpu().numpy()
+            thr = np.full(batch, 0.5, np.float32)
+            t0 = time.perf_counter()
+            for l in layers:
+                c, ih, iw, kn, kw, kh, p, s = l["shape"]
+                xh = ref.conv(TNN, xh, thr, O.aligned_copy(l["qw"].cpu().numpy()), kn, kh, kw, p, s, 0.5)
+            row["cpu_ms"] = round((time.perf_counter() - t0) * 1e3, 1)
+            row["bit_exact_vs_reference"] = bool(y.cpu().numpy().tobytes() == np.ascontiguousarray(xh).tobytes())
+        net.close()
+        out[net_t["name"]] = row
+        del layers, x, y
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -435,6 +486,7 @@ def main():
             "tbn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, TBN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 3),
             "btn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, BTN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 4),
             "tnn_resnet18_like_b32_e2e": e2e_latency(torch, lib, 32),
+            "reference_e2e_networks_b8": reference_networks(torch, lib),
             "tnn_resnet18_like_other_batches": {"b%d" % b: e2e_latency(torch, lib, b, cpu=False) for b in (1, 8, 128)},
         }
 
