@@ -312,6 +312,42 @@ def e2e_latency(torch, lib, batch, reps=10, cpu=True):
     return out
 
 
+def reference_gemm_sweep(torch, lib, reps=10):
+    """the sweep of the reference's GEMM driver, m = n in {32 .. 4096}, p = 8 m (src/timing_gemm.c:90-97), alpha = 1 as
+    tnns_gemm (src/tnns/tnns_cpu_mm_p2.c:123): device-resident operands, the engine the library picks, against the
+    reference on one host core"""
+    import numpy as np
+    from fastertnn_amd import TNN
+    from oracle import ftnn_oracle as O
+    out = {}
+    for m in (32, 64, 128, 256, 512, 1024, 2048, 4096):
+        p = 8 * m
+        kw = p // 64
+        a = ternary_operand(torch, lib, m, p, seed=20 + m)
+        b = ternary_operand(torch, lib, m, p, seed=21 + m)
+        y = torch.empty((m, m, 1, 1), dtype=torch.float32, device="cuda")
+        need = lib.mm_scratch_bytes(lib.ENGINE_AUTO, TNN, m, 1, 1, m, kw)
+        scratch = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+
+        def run():
+            lib.mm_engine(lib.ENGINE_AUTO, TNN, a, b, m, 1, 1, m, kw, 1.0, out=y, scratch=scratch)
+        for _ in range(3):
+            run()
+        t = sorted(event_times(torch, run, reps))[reps // 2]
+        row = {"engine": lib.ENGINE_NAMES[lib.select_engine(TNN, m, 1, 1, m, kw)], "device_ms": round(t, 4),
+               "gmacs": round(float(m) * m * p / t / 1e6, 1)}
+        if O.Reference.available():
+            ref = O.Reference()
+            ah, bh = O.aligned_copy(a.cpu().numpy()), O.aligned_copy(b.cpu().numpy())
+            t0 = time.perf_counter()
+            want = ref.mm(TNN, ah, bh, m, 1, 1, m, kw, 1.0)
+            row["cpu_ms"] = round((time.perf_counter() - t0) * 1e3, 3)
+            row["bit_exact_vs_reference"] = bool(y.cpu().numpy().tobytes() == np.ascontiguousarray(want).tobytes())
+        out["m%d" % m] = row
+        del a, b, y, scratch
+    return out
+
+
 def reference_networks(torch, lib, batch=8, reps=5):
     """the networks of the reference's e2e mode that chain shape to shape (include/timing/shapes_e2e.h, kept as
     data in tests/golden/reference_shape_tables.json), at the reference's batch of 8 (src/timing_layers.c:46):
@@ -486,6 +522,7 @@ def main():
             "tbn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, TBN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 3),
             "btn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, BTN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 4),
             "tnn_resnet18_like_b32_e2e": e2e_latency(torch, lib, 32),
+            "reference_gemm_sweep": reference_gemm_sweep(torch, lib),
             "reference_e2e_networks_b8": reference_networks(torch, lib),
             "tnn_resnet18_like_other_batches": {"b%d" % b: e2e_latency(torch, lib, b, cpu=False) for b in (1, 8, 128)},
         }
