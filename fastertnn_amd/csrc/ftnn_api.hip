@@ -356,9 +356,10 @@ int ftnn_mm(int type, const int64_t* d_a, const int64_t* d_b, int N, int OH, int
 // over the CUs; below that the vector-ALU kernel is faster.
 static int select_engine(int type, int64_t M, int KN, int Kw) {
     (void)type;
-    const int64_t tiles = ((M + 255) / 256) * ((KN + 255) / 256);
+    // measured on MI355X: from about 5 GMAC the two expansions and the matrix-core kernel (128 x 128 tiles
+    // while 256 x 256 ones would leave compute units idle) take less time than the vector-ALU kernel
     const double lane_macs = (double)M * KN * 64.0 * Kw;
-    if (lane_macs >= 1.2e10 && tiles >= 48 && KN >= 128 && 64LL * Kw < (1LL << 24)) return FTNN_ENGINE_MFMA_F4;
+    if (lane_macs >= 5e9 && KN >= 128 && 64LL * Kw < (1LL << 24)) return FTNN_ENGINE_MFMA_F4;
     return FTNN_ENGINE_VALU;
 }
 

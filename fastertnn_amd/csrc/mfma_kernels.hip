@@ -36,9 +36,17 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kKF = 2;   // fragments per row-block and step
 constexpr int kNS = 4;   // LDS ring depth
-constexpr int kFR = 16 * kKF;            // fragments per step: (8 P + 8 Q row-blocks) x kKF
-constexpr int kFW = kFR / 4;             // fragments staged by one wavefront per step
-constexpr size_t kLdsBytes = (size_t)kNS * kFR * 1024;
+// A workgroup of 2 x 2 wavefronts computes (64 WT) x (64 WT) results, a wavefront WT x WT blocks of 32 x 32:
+// WT = 4 for problems with enough 256 x 256 tiles to fill the chip, WT = 2 (128 x 128) below that.
+template <int WT>
+struct Tile {
+    static constexpr int RB = 2 * WT;             // row-blocks per operand side
+    static constexpr int FR = 2 * RB * kKF;       // fragments per step: (RB P + RB Q row-blocks) x kKF
+    static constexpr int FW = FR / 4;             // fragments staged by one wavefront per step
+    static constexpr int NL = 2 * WT;             // LDS reads per wavefront and k fragment
+    static constexpr size_t lds_bytes = (size_t)kNS * FR * 1024;
+    static_assert(FW == NL && (WT * WT) % NL == 0, "one staged fragment and WT/2 multiplies per LDS read");
+};
 
 // ------------------------------------------------------------------ expansion
 // grid (row-blocks, groups), block 256: thread = (row r = t%32, dword pair dq = t/32).
@@ -138,33 +146,34 @@ __device__ __forceinline__ void dma16(const uint4* gsrc, uint32_t lds_byte_addr)
 // The epilogue computes r = acc - bias, then PReLU in the reference's form for the type:
 // form 0 "f = r; if (f <= 0) f *= alpha" (mm_p2_final_tnn_avx2.c:204-208), form 1
 // "r >= 0 ? r : alpha * r" (mm_p2_final_tbn_avx2.c:73).
-template <bool F4, bool SWAP>
+template <bool F4, bool SWAP, int WT>
 __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, const uint4* __restrict__ Qf,
                                               float* __restrict__ Y, int M, int KN, int OHW, int KB,
                                               int bias, int form, float alpha) {
     extern __shared__ uint4 lds[];   // kNS buffers of kFR KiB
     typedef typename Acc<F4>::type acc_t;
+    constexpr int RB = Tile<WT>::RB, kFR = Tile<WT>::FR, kFW = Tile<WT>::FW, NL = Tile<WT>::NL;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wy = wave >> 1, wx = wave & 1;
     const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN;
-    const int prb0 = blockIdx.x * 8, qrb0 = blockIdx.y * 8;
+    const int prb0 = blockIdx.x * RB, qrb0 = blockIdx.y * RB;
     const int prbmax = (prow + 31) / 32 - 1, qrbmax = (qrow + 31) / 32 - 1;
-    acc_t acc[4][4];
+    acc_t acc[WT][WT];
 #pragma unroll
-    for (int a = 0; a < 4; a++)
+    for (int a = 0; a < WT; a++)
 #pragma unroll
-        for (int b = 0; b < 4; b++)
+        for (int b = 0; b < WT; b++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[a][b][e] = 0;
 
-    // fragment f of a step: side f / (8*kKF) (0 = P, 1 = Q), row-block (f / kKF) % 8, k fragment
+    // fragment f of a step: side f / (RB*kKF) (0 = P, 1 = Q), row-block (f / kKF) % RB, k fragment
     // f % kKF; row-blocks past the operand are clamped (their results are never stored)
     const uint4* src[kFW];
 #pragma unroll
     for (int i = 0; i < kFW; i++) {
         const int f = wave * kFW + i;
-        const int side = f / (8 * kKF), rbi = (f / kKF) % 8, kbi = f % kKF;
+        const int side = f / (RB * kKF), rbi = (f / kKF) % RB, kbi = f % kKF;
         const uint4* base = side == 0 ? Pf + ((size_t)min(prb0 + rbi, prbmax) * KB + kbi) * 64
                                       : Qf + ((size_t)min(qrb0 + rbi, qrbmax) * KB + kbi) * 64;
         src[i] = base + lane;
@@ -176,18 +185,22 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
 #pragma unroll
         for (int i = 0; i < kFW; i++) dma16(src[i] + (size_t)step * kKF * 64, dst + i * 1024);
     };
-    uint4 fa[2][4], fb[2][4];
+    uint4 fa[2][WT], fb[2][WT];
     // one LDS read of fragment k of buffer `buf` into register set `set`, in the order the MFMAs
-    // consume them: i = 0: fa0, 1..4: fb0..fb3, 5..7: fa1..fa3
+    // consume them: i = 0: fa0, 1..WT: fb0..fb(WT-1), then fa1..fa(WT-1)
     auto ldone = [&](int buf, int k, int set, int i) {
         const uint4* L = lds + (size_t)buf * kFR * 64;
-        if (i == 0) fa[set][0] = L[((wy * 4 + 0) * kKF + k) * 64 + lane];
-        else if (i <= 4) fb[set][i - 1] = L[((8 + wx * 4 + (i - 1)) * kKF + k) * 64 + lane];
-        else fa[set][i - 4] = L[((wy * 4 + (i - 4)) * kKF + k) * 64 + lane];
+        if (i == 0) fa[set][0] = L[((wy * WT + 0) * kKF + k) * 64 + lane];
+        else if (i <= WT) fb[set][i - 1] = L[((RB + wx * WT + (i - 1)) * kKF + k) * 64 + lane];
+        else fa[set][i - WT] = L[((wy * WT + (i - WT)) * kKF + k) * 64 + lane];
     };
+    // the WT/2 multiplies that go with LDS read i
     auto mfma2 = [&](int set, int i) {
-        mfma<F4>(acc[(2 * i) / 4][(2 * i) % 4], fa[set][(2 * i) / 4], fb[set][(2 * i) % 4]);
-        mfma<F4>(acc[(2 * i + 1) / 4][(2 * i + 1) % 4], fa[set][(2 * i + 1) / 4], fb[set][(2 * i + 1) % 4]);
+#pragma unroll
+        for (int j = 0; j < WT / 2; j++) {
+            const int m = (WT / 2) * i + j;
+            mfma<F4>(acc[m / WT][m % WT], fa[set][m / WT], fb[set][m % WT]);
+        }
     };
 
     // prologue: the first kNS stages in flight, wait for stage 0 only
@@ -198,7 +211,7 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 8; i++) ldone(0, 0, 0, i);
+    for (int i = 0; i < NL; i++) ldone(0, 0, 0, i);
 
     auto step_body = [&](int s, auto full_tag) {
         constexpr bool FULL = decltype(full_tag)::value;   // FULL: s + kNS < nstep
@@ -207,7 +220,7 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
             const int set = k & 1;
             if (k + 1 < kKF) {
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
+                for (int i = 0; i < NL; i++) {
                     ldone(s % kNS, k + 1, set ^ 1, i);
                     mfma2(set, i);
                     __builtin_amdgcn_sched_barrier(0);
@@ -222,13 +235,8 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
                 const bool do_ld = FULL || s + 1 < nstep;
                 const uint32_t dst = lds0 + (uint32_t)(s % kNS) * (kFR * 1024) + wave * (kFW * 1024);
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    if (FULL) {
-#pragma unroll
-                        for (int j = 0; j < kFW / 8; j++)
-                            dma16(src[i * (kFW / 8) + j] + (size_t)(s + kNS) * kKF * 64,
-                                  dst + (i * (kFW / 8) + j) * 1024);
-                    }
+                for (int i = 0; i < NL; i++) {
+                    if (FULL) dma16(src[i] + (size_t)(s + kNS) * kKF * 64, dst + i * 1024);
                     if (do_ld) ldone((s + 1) % kNS, 0, set ^ 1, i);
                     mfma2(set, i);
                     __builtin_amdgcn_sched_barrier(0);
@@ -244,11 +252,11 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
     // SWAP = false is only launched for OHW == 1 (row-major m x n result).
     const bool le_form = form == 0;
 #pragma unroll
-    for (int a = 0; a < 4; a++)
+    for (int a = 0; a < WT; a++)
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
-            const int q = (qrb0 + wx * 4 + b) * 32 + (lane & 31);
-            const int pbase = (prb0 + wy * 4 + a) * 32 + 4 * (lane >> 5);
+        for (int b = 0; b < WT; b++) {
+            const int q = (qrb0 + wx * WT + b) * 32 + (lane & 31);
+            const int pbase = (prb0 + wy * WT + a) * 32 + 4 * (lane >> 5);
             size_t qoff;
             if (SWAP) {   // q = i is fixed per block: split it into (image, pixel) once
                 const int img = q / OHW;
@@ -535,19 +543,40 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
     });
 }
 
+// tiles of 256 x 256 below which the 128 x 128 kernel is used (FTNN_MFMA_SMALL_BELOW: tuning aid)
+inline int64_t mfma_small_tile_below() {
+    static const int64_t v = []() {
+        const char* e = getenv("FTNN_MFMA_SMALL_BELOW");
+        return e ? (int64_t)atoll(e) : (int64_t)160;
+    }();
+    return v;
+}
+
+template <bool F4, bool SWAP, int WT>
+hipError_t launch_gemm_tile(const uint4* Pf, const uint4* Qf, float* Y, int M, int KN, int OHW, int KB,
+                            int bias, int form, float alpha, hipStream_t st) {
+    auto kern = k_mfma<F4, SWAP, WT>;
+    constexpr size_t lds_bytes = Tile<WT>::lds_bytes;
+    // the opt-in to more than 64 KiB of dynamic LDS is per kernel; done once, thread-safe
+    static const hipError_t configured = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (configured != hipSuccess) return configured;
+    const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN, edge = 64 * WT;
+    dim3 grid((prow + edge - 1) / edge, (qrow + edge - 1) / edge);
+    if (grid.y > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, st, Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha);
+    return hipGetLastError();
+}
+
 template <bool F4, bool SWAP>
 hipError_t launch_gemm(const uint4* Pf, const uint4* Qf, float* Y, int M, int KN, int OHW, int KB,
                        int bias, int form, float alpha, hipStream_t st) {
-    auto kern = k_mfma<F4, SWAP>;
-    // the opt-in to more than 64 KiB of dynamic LDS is per kernel; done once, thread-safe
-    static const hipError_t configured = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
-    if (configured != hipSuccess) return configured;
-    const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN;
-    dim3 grid((prow + 255) / 256, (qrow + 255) / 256);
-    if (grid.y > 65535) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(kern, grid, dim3(256), kLdsBytes, st, Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha);
-    return hipGetLastError();
+    // 256 x 256 tiles re-read the operands least, but a problem must have enough of them for the chip's
+    // 256 compute units; below that, 128 x 128 tiles (two workgroups fit a compute unit)
+    const int64_t big = (((int64_t)M + 255) / 256) * ((KN + 255) / 256);
+    bool small = big < mfma_small_tile_below();
+    return small ? launch_gemm_tile<F4, SWAP, 2>(Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha, st)
+                 : launch_gemm_tile<F4, SWAP, 4>(Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha, st);
 }
 
 template <bool F4>

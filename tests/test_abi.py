@@ -89,7 +89,8 @@ def test_engine_selection_and_scratch_sizes_need_no_device():
     assert lib.select_engine(0, 2048, 1, 1, 2048, 256) == lib.ENGINE_MFMA_F4
     assert lib.select_engine(0, 1, 56, 56, 256, 36) == lib.ENGINE_VALU
     assert lib.select_engine(0, 32, 56, 56, 64, 9) == lib.ENGINE_VALU
-    assert lib.select_engine(0, 512, 1, 1, 512, 512) == lib.ENGINE_VALU          # too few tiles
+    assert lib.select_engine(0, 1024, 1, 1, 1024, 128) == lib.ENGINE_MFMA_F4      # the mid sizes of the reference's sweep too
+    assert lib.select_engine(0, 512, 1, 1, 512, 64) == lib.ENGINE_VALU            # too little work for three launches
     # fp32 accumulation of fp4 products is exact only below 2^24 lanes: never chosen beyond
     assert lib.select_engine(0, 4096, 1, 1, 4096, 1 << 18) == lib.ENGINE_VALU
     assert lib.mm_scratch_bytes(lib.ENGINE_VALU, 0, 8192, 1, 1, 8192, 512) == 0

@@ -74,6 +74,27 @@ def test_row_major_gemm_all_types(hip, oracle, typ, mnk):
             assert got.tobytes() == want.tobytes(), "engine %d alpha %g" % (eng, alpha)
 
 
+@pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
+@pytest.mark.parametrize("shape", [(3333, 1, 1, 3100, 4), (5, 29, 29, 2700, 12)], ids=["row_major", "nchw"])
+def test_matrix_core_engines_with_256x256_tiles(hip, oracle, typ, shape):
+    """the matrix-core kernel works on 128 x 128 tiles while a problem has few of them and on 256 x 256
+    tiles from 160 of those on; the cases above are all of the first kind, these are of the second
+    (ragged in both directions, row-major and NCHW stores)"""
+    n, oh, ow, kn, kw = shape
+    m = n * oh * ow
+    assert ((m + 255) // 256) * ((kn + 255) // 256) >= 160
+    rng = np.random.default_rng(77 + typ + kw)
+    at, wt = act_is_ternary(typ), weight_is_ternary(typ)
+    a = rng.integers(-2 ** 63, 2 ** 63, size=m * kw * (2 if at else 1), dtype=np.int64)
+    b = rng.integers(-2 ** 63, 2 ** 63, size=kn * kw * (2 if wt else 1), dtype=np.int64)
+    ku = 64 * kw - 3
+    want = oracle.mm(typ, a, b, n, oh, ow, kn, kw, 0.5, ku)
+    a_d, b_d = _dev(a), _dev(b)
+    for eng in (hip.ENGINE_MFMA_I8, hip.ENGINE_MFMA_F4):
+        got = hip.mm_engine(eng, typ, a_d, b_d, n, oh, ow, kn, kw, 0.5, ku).cpu().numpy()
+        assert got.tobytes() == want.tobytes(), "engine %d" % eng
+
+
 def test_lanes_flagged_zero_and_negative_count_as_zero(hip, oracle):
     """a lane with both its sign and its zero bit set is zero in the reference's formula
     (za|zb masks it); the expanded operands must agree"""
