@@ -38,6 +38,9 @@ static int check_conv_shape(int N, int C, int H, int W, int H_pad, int W_pad, in
         return fail(FTNN_EINVAL, "kernel %dx%d larger than padded input %dx%d", kH, kW,
                     H + 2 * H_pad, W + 2 * W_pad);
     if (N > 65535) return fail(FTNN_EINVAL, "batch %d above the supported 65535", N);
+    // pixel indices within one image plane are 32-bit in the kernels (27 of them in one store offset)
+    if (((int64_t)H + 2 * H_pad) * ((int64_t)W + 2 * W_pad) > 0x3ffffffLL)
+        return fail(FTNN_EINVAL, "padded image plane above the supported 2^26 pixels");
     *OH = out_dim(H, H_pad, kH, H_stride);
     *OW = out_dim(W, W_pad, kW, W_stride);
     return FTNN_OK;

@@ -492,12 +492,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
                 if (q < M) {
                     if (kn0 + 32 * a + 32 <= KN) {   // whole block inside: no per-kernel checks
 #pragma unroll
-                        for (int e = 0; e < 16; e++) yq[(size_t)((8 * (e >> 2) + (e & 3)) * OHW)] = vals[e];
+                        for (int e = 0; e < 16; e++) yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = vals[e];
                     } else {
 #pragma unroll
                         for (int e = 0; e < 16; e++) {
                             const int p = kn0 + 32 * a + 8 * (e >> 2) + 4 * h + (e & 3);
-                            if (p < KN) yq[(size_t)((8 * (e >> 2) + (e & 3)) * OHW)] = vals[e];
+                            if (p < KN) yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = vals[e];
                         }
                     }
                 }

@@ -77,3 +77,70 @@ def test_resnet_stage_layers_batch32(hip, oracle, typ):
         want = oracle.conv(typ, x[n:n + 1].cpu().numpy(), thr[n:n + 1].cpu().numpy(), qw.cpu().numpy(), c, 3, 3,
                            1, 1, 0.5)
         assert y[n:n + 1].cpu().numpy().tobytes() == want.tobytes()
+
+
+def _rand_words(torch, count, seed):
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    return torch.randint(-2 ** 62, 2 ** 62, (count,), generator=g, device="cuda", dtype=torch.int64)
+
+
+def test_row_major_result_beyond_2_32_elements(hip, oracle):
+    """66000 x 65600 results (17 GB): offsets into the result need more than 32 bits.  All three engines agree
+    on every element, and rows on either side of the 2^31- and 2^32-element marks are bit-exact against the oracle"""
+    import torch
+    m, n, kw = 66000, 65600, 4
+    assert m * n > 2 ** 32
+    a, b = _rand_words(torch, m * 2 * kw, 1), _rand_words(torch, n * 2 * kw, 2)
+    ref = None
+    for eng in (hip.ENGINE_VALU, hip.ENGINE_MFMA_F4, hip.ENGINE_MFMA_I8):
+        print("engine", eng, flush=True)
+        y = torch.full((m, n, 1, 1), float("nan"), dtype=torch.float32, device="cuda")
+        hip.mm_engine(eng, TNN, a, b, m, 1, 1, n, kw, 0.5, out=y)
+        if ref is None:
+            ref = y
+            rows = [0, 2 ** 31 // n, 2 ** 31 // n + 1, 2 ** 32 // n, 2 ** 32 // n + 1, m - 1]
+            ah = a.view(m, 2 * kw)[rows].cpu().numpy()
+            want = oracle.mm(TNN, np.ascontiguousarray(ah).reshape(-1), b.cpu().numpy(), len(rows), 1, 1, n, kw, 0.5)
+            assert y.view(m, n)[rows].cpu().numpy().tobytes() == want.tobytes()
+        else:
+            assert torch.equal(y, ref), "engine %d" % eng
+            del y
+
+
+def test_nchw_results_beyond_2_32_elements(hip, oracle):
+    """1050 images x 1000 kernels x 64 x 64 pixels (17 GB) from a 3x3 layer: both layer engines and the GEMM
+    engines behind packed rows agree on every element; the first, the last and the images around the 2^31- and
+    2^32-element marks are bit-exact against the oracle"""
+    import torch
+    n, c, hw, kn = 1050, 64, 64, 1000
+    assert n * kn * hw * hw > 2 ** 32
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    x = torch.randn((n, c, hw, hw), generator=g, device="cuda")
+    thr = torch.full((n,), 0.5, device="cuda")
+    from fastertnn_amd import synth
+    w = synth.ternary(9, (kn, c, 3, 3))
+    qw_h = oracle.pack_weights(w, np.full(kn, 0.5, np.float32), True)
+    qw = torch.from_numpy(qw_h).cuda()
+    per_img = kn * hw * hw
+    imgs = [0, 2 ** 31 // per_img, 2 ** 31 // per_img + 1, 2 ** 32 // per_img, 2 ** 32 // per_img + 1, n - 1]
+    ref = None
+    for eng in (hip.ENGINE_MFMA_F4, hip.ENGINE_VALU):
+        print("layer engine", eng, flush=True)
+        y = torch.full((n, kn, hw, hw), float("nan"), dtype=torch.float32, device="cuda")
+        hip.conv(TNN, x, thr, qw, kn, 3, 3, 1, 1, 0.5, out=y, engine=eng)
+        if ref is None:
+            ref = y
+            want = oracle.conv(TNN, x[imgs].cpu().numpy(), np.full(len(imgs), 0.5, np.float32), qw_h, kn, 3, 3, 1, 1, 0.5)
+            assert y[imgs].cpu().numpy().tobytes() == np.ascontiguousarray(want).tobytes()
+        else:
+            assert torch.equal(y, ref), "layer engine %d" % eng
+            del y
+    rows = hip.quantize_im2row(x, thr, 3, 3, 1, 1, True)
+    for eng in (hip.ENGINE_MFMA_F4, hip.ENGINE_MFMA_I8):
+        print("gemm engine", eng, flush=True)
+        y = torch.full((n, kn, hw, hw), float("nan"), dtype=torch.float32, device="cuda")
+        hip.mm_engine(eng, TNN, rows, qw, n, hw, hw, kn, 9, 0.5, out=y)
+        assert torch.equal(y, ref), "gemm engine %d" % eng
+        del y
