@@ -312,6 +312,20 @@ def e2e_latency(torch, lib, batch, reps=10, cpu=True):
     return out
 
 
+def valu_probe():
+    """the measured issue rate of v_bcnt_u32_b32 over the whole chip (fastertnn_amd/csrc/probe_valu.hip, a child
+    process): what the nominal 39.3 T lane-op/s of the vector-ALU roofline comes to at the clock the chip holds"""
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fastertnn_amd", "probe_valu")
+    if not os.path.exists(exe):
+        return {"skipped": "fastertnn_amd/probe_valu is not built"}
+    p = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    for line in p.stdout.splitlines():
+        if line.startswith("{"):
+            return json.loads(line)
+    return {"failed": p.stdout[-200:]}
+
+
 def reference_gemm_sweep(torch, lib, reps=10):
     """the sweep of the reference's GEMM driver, m = n in {32 .. 4096}, p = 8 m (src/timing_gemm.c:90-97), alpha = 1 as
     tnns_gemm (src/tnns/tnns_cpu_mm_p2.c:123): device-resident operands, the engine the library picks, against the
@@ -522,6 +536,7 @@ def main():
             "tbn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, TBN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 3),
             "btn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, BTN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 4),
             "tnn_resnet18_like_b32_e2e": e2e_latency(torch, lib, 32),
+            "valu_popcount_probe": valu_probe(),
             "reference_gemm_sweep": reference_gemm_sweep(torch, lib),
             "reference_e2e_networks_b8": reference_networks(torch, lib),
             "tnn_resnet18_like_other_batches": {"b%d" % b: e2e_latency(torch, lib, b, cpu=False) for b in (1, 8, 128)},

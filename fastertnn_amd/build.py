@@ -6,6 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libftnn_hip.so")
+PROBE = os.path.join(HERE, "probe_valu")   # stand-alone measurement aid (vector-ALU popcount issue rate)
 SOURCES = ["ftnn_api.hip", "pack_kernels.hip", "mm_kernels.hip", "mfma_kernels.hip", "ftnn_net.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
@@ -60,7 +61,18 @@ def build_library(verbose=False):
             print(out)
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB]
     subprocess.run(cmd, check=True)
+    build_probe()
     return LIB
+
+
+def build_probe():
+    """the popcount issue-rate probe bench.py runs beside the GEMM (its own executable, not part of the library)"""
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", os.path.join(CSRC, "probe_valu.hip"), "-o", PROBE]
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("hipcc failed on probe_valu.hip:\n%s" % p.stdout)
+    return PROBE
 
 
 if __name__ == "__main__":
