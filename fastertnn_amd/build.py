@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libftnn_hip.so")
 PROBE = os.path.join(HERE, "probe_valu")   # stand-alone measurement aid (vector-ALU popcount issue rate)
-SOURCES = ["ftnn_api.hip", "pack_kernels.hip", "mm_kernels.hip", "mfma_kernels.hip", "ftnn_net.hip"]
+SOURCES = ["ftnn_api.hip", "pack_kernels.hip", "mm_kernels.hip", "mfma_kernels.hip", "stem_kernels.hip", "ftnn_net.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -204,6 +204,12 @@ int conv_f4_expanded(int type, const float* d_x, const float* d_thr, const void*
         // few channels: several taps per 64-lane word, materialised per output pixel; the layer is then a 1x1
         // layer with Kd words per pixel over the OH x OW output pixels
         if (!d_x) return fail(FTNN_EINVAL, "a few-channel layer takes fp32 input");
+        static const bool fused_off = getenv("FTNN_NO_FUSED_STEM") != nullptr;   // tuning aid: the two-kernel form
+        if (stem_f4_lds_bytes(C, KH, KW, H_stride, W_stride) > 0 && !fused_off) {
+            e = launch_stem_f4(type, d_x, d_thr, d_wf, N, C, H, W, KN, KH, KW, H_pad, W_pad, H_stride, W_stride,
+                               prelu_alpha, d_y, st, qo);
+            return e == hipSuccess ? FTNN_OK : hip_fail(e, "fp4 first-layer launch");
+        }
         int T, Kd;
         dense_applies(C, KH, KW, &T, &Kd);
         void* d_a4 = static_cast<char*>(d_p4) + dense_f4_pq_bytes(N, H, W);

@@ -62,6 +62,32 @@ __device__ __forceinline__ uint32_t quant_nibble(float v, float t, bool ternary,
     return r;
 }
 
+// The ternary hand-over without compares, for the slopes and thresholds layers use (anything else takes
+// quant_nibble on the PReLU result).  Both PReLU forms leave r > 0 as it is and turn r <= 0 into r * alpha <= 0, so
+// for alpha >= 0 and t >= 0: PReLU(r) > t <=> r > t, and PReLU(r) < -t <=> r * alpha < -t (r * alpha is the very
+// product PReLU forms; for r > 0 it is >= 0 >= -t).  r is an integer: with 2^-20 <= alpha <= 2^20 (or alpha = 0) and
+// t <= 2^40, a difference r - t or -(r * alpha) - t that is positive is at least 2^-44, so 2^60 times it clamps to
+// exactly 1, and one that is not positive clamps to +0.  The result is +1, -1 or +0 as a float, which
+// v_cvt_scalef32_pk_fp4_f32 turns into the E2M1 nibbles 0x2, 0xA, 0x0, two values per instruction.
+__device__ __forceinline__ bool tern_direct_applies(float alpha, float t) {
+    return (alpha == 0.0f || (alpha >= 0x1p-20f && alpha <= 0x1p20f)) && t >= 0.0f && t <= 0x1p40f;
+}
+__device__ __forceinline__ float tern_value_direct(float r, float alpha, float t_big /* t * 2^60 */) {
+    const float pos = __builtin_amdgcn_fmed3f(__builtin_fmaf(r, 0x1p60f, -t_big), 0.0f, 1.0f);
+    const float neg = __builtin_amdgcn_fmed3f(__builtin_fmaf(r * alpha, -0x1p60f, -t_big), 0.0f, 1.0f);
+    return pos - neg;
+}
+// eight values out of {+1, -1, +0} -> one dword of E2M1 nibbles, value k in nibble k
+__device__ __forceinline__ uint32_t pack_fp4x8(float z0, float z1, float z2, float z3, float z4, float z5, float z6,
+                                               float z7) {
+    uint32_t d = 0u;
+    d = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(d, z0, z1, 1.0f, 0);
+    d = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(d, z2, z3, 1.0f, 1);
+    d = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(d, z4, z5, 1.0f, 2);
+    d = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(d, z6, z7, 1.0f, 3);
+    return d;
+}
+
 // record a failure text for ftnn_last_error(); returns `code`
 int fail(int code, const char* fmt, ...);
 
@@ -101,6 +127,12 @@ hipError_t launch_dense_weights(bool ternary, const int64_t* d_qw, int KN, int C
 // dense_f4_pq_bytes), then string T taps per 64-lane word into A4[n][Kd][output pixel][32 bytes] (d_a4), the
 // operand of launch_conv_f4 for a 1x1 layer with C_pack = Kd over the OH x OW output pixels
 bool dense_f4_applies(int C, int KH, int KW);
+// stem_kernels.hip: the same layer in one kernel (fp32 input -> result, the rows never stored) where its input
+// patch fits the LDS: bytes of LDS it needs, 0 = does not apply
+int64_t stem_f4_lds_bytes(int C, int KH, int KW, int H_stride, int W_stride);
+hipError_t launch_stem_f4(int type, const float* d_x, const float* d_thr, const void* d_wf, int N, int C, int H,
+                          int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride, int W_stride,
+                          float alpha, float* d_y, hipStream_t st, const QuantOut& qo);
 int64_t dense_f4_pq_bytes(int N, int H, int W);
 hipError_t launch_dense_rows_f4(bool ternary, const float* d_x, const float* d_thr, int N, int C, int H, int W,
                                 int H_pad, int W_pad, int kH, int kW, int H_stride, int W_stride, void* d_pq,

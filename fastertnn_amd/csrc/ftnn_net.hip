@@ -109,6 +109,13 @@ ftnn_net_t* ftnn_net_create(int batch, int n_layers, const ftnn_layer_t* layers)
         net->layers.push_back(L);
         net->OH.push_back(out_dim(L.H, L.pad, L.KH, L.stride));
         net->OW.push_back(out_dim(L.W, L.pad, L.KW, L.stride));
+        // the same size limits as a single layer call
+        if (((int64_t)L.H + 2 * L.pad) * ((int64_t)L.W + 2 * L.pad) > 0x3ffffffLL ||
+            (int64_t)batch * net->OH[i] * net->OW[i] > 0x7fffff00LL) {
+            fail(FTNN_EINVAL, "layer %d: image plane above 2^26 pixels or more than 2^31 output rows", i);
+            ftnn_net_destroy(net);
+            return nullptr;
+        }
         net->out_elems = (int64_t)batch * L.KN * net->OH[i] * net->OW[i];
     }
     // engine of every layer, then the buffers the chain needs between them

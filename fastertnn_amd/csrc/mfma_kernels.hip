@@ -49,57 +49,70 @@ struct Tile {
 };
 
 // ------------------------------------------------------------------ expansion
-// grid (row-blocks, groups), block 256: thread = (row r = t%32, dword pair dq = t/32).
+// grid (row-blocks, groups / 4), block 256: thread = (row r = t%32, dword pair dq = t/32).
 // A group is 4 words (256 lanes) of a packed row: 16 dwords (8 sign, 8 zero) for ternary
 // rows, 8 dwords for binary rows.  Rows past `rows` expand to zeros.
 template <bool F4, bool TERN>
 __global__ __launch_bounds__(256) void k_expand(const uint32_t* __restrict__ P, int rows, int G,
                                                 uint4* __restrict__ out) {
-    const int rb = blockIdx.x, g = blockIdx.y, t = threadIdx.x;
+    // a workgroup expands kGPB adjacent groups of its 32 rows: 256 contiguous bytes of each ternary row, so
+    // that both halves of a 128-byte line are consumed by the same workgroup, with all loads issued up front
+    constexpr int kGPB = 4;
+    const int rb = blockIdx.x, g0 = blockIdx.y * kGPB, t = threadIdx.x;
     const int r = t & 31, dq = t >> 5;
     const int row = min(rb * 32 + r, rows - 1);
     const bool live = rb * 32 + r < rows;
-    uint32_t s, nz;
-    if (TERN) {
-        const uint32_t* src = P + ((size_t)row * G + g) * 16;
-        nz = live ? ~src[8 + dq] : 0u;
-        s = src[dq] & nz;   // a lane flagged zero is zero whatever its sign bit says
-    } else {
-        const uint32_t* src = P + ((size_t)row * G + g) * 8;
-        nz = live ? 0xffffffffu : 0u;
-        s = src[dq] & nz;
-    }
-    if (F4) {
-        // fragment = one 64-lane word: dword dq&1 is its k half; nibble = sign<<3 | nonzero<<1
-        uint4* frag = out + ((size_t)rb * (G * 4) + (g * 4 + (dq >> 1))) * 64;
-        uint32_t o[4];
+    uint32_t sv[kGPB], zv[kGPB];
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            uint32_t a = (s >> (8 * q)) & 0xffu, b = (nz >> (8 * q)) & 0xffu;
-            a = (a | (a << 12)) & 0x000F000Fu;
-            a = (a | (a << 6)) & 0x03030303u;
-            a = (a | (a << 3)) & 0x11111111u;
-            b = (b | (b << 12)) & 0x000F000Fu;
-            b = (b | (b << 6)) & 0x03030303u;
-            b = (b | (b << 3)) & 0x11111111u;
-            o[q] = (a << 3) | (b << 1);
+    for (int i = 0; i < kGPB; i++) {
+        const int g = min(g0 + i, G - 1);
+        if (TERN) {
+            const uint32_t* src = P + ((size_t)row * G + g) * 16;
+            sv[i] = src[dq];
+            zv[i] = src[8 + dq];
+        } else {
+            sv[i] = P[((size_t)row * G + g) * 8 + dq];
+            zv[i] = 0u;
         }
-        frag[(dq & 1) * 32 + r] = make_uint4(o[0], o[1], o[2], o[3]);
-    } else {
-        // fragment = one 32-lane dword: its two 16-lane halves are the k halves
-        uint4* frag = out + ((size_t)rb * (G * 8) + (g * 8 + dq)) * 64;
+    }
 #pragma unroll
-        for (int half = 0; half < 2; half++) {
-            const uint32_t sh = (s >> (16 * half)) & 0xffffu, nh = (nz >> (16 * half)) & 0xffffu;
+    for (int i = 0; i < kGPB; i++) {
+        const int g = g0 + i;
+        if (g >= G) break;
+        const uint32_t nz = live ? ~zv[i] : 0u;
+        const uint32_t s = sv[i] & nz;   // a lane flagged zero is zero whatever its sign bit says
+        if (F4) {
+            // fragment = one 64-lane word: dword dq&1 is its k half; nibble = sign<<3 | nonzero<<1
+            uint4* frag = out + ((size_t)rb * (G * 4) + (g * 4 + (dq >> 1))) * 64;
             uint32_t o[4];
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                // 4 bits -> 4 byte LSBs: bit i lands on bit 8i, no carries
-                const uint32_t sb = (((sh >> (4 * q)) & 15u) * 0x204081u) & 0x01010101u;
-                const uint32_t nb = (((nh >> (4 * q)) & 15u) * 0x204081u) & 0x01010101u;
-                o[q] = nb | (sb * 0xffu);
+                uint32_t a = (s >> (8 * q)) & 0xffu, b = (nz >> (8 * q)) & 0xffu;
+                a = (a | (a << 12)) & 0x000F000Fu;
+                a = (a | (a << 6)) & 0x03030303u;
+                a = (a | (a << 3)) & 0x11111111u;
+                b = (b | (b << 12)) & 0x000F000Fu;
+                b = (b | (b << 6)) & 0x03030303u;
+                b = (b | (b << 3)) & 0x11111111u;
+                o[q] = (a << 3) | (b << 1);
             }
-            frag[half * 32 + r] = make_uint4(o[0], o[1], o[2], o[3]);
+            frag[(dq & 1) * 32 + r] = make_uint4(o[0], o[1], o[2], o[3]);
+        } else {
+            // fragment = one 32-lane dword: its two 16-lane halves are the k halves
+            uint4* frag = out + ((size_t)rb * (G * 8) + (g * 8 + dq)) * 64;
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+                const uint32_t sh = (s >> (16 * half)) & 0xffffu, nh = (nz >> (16 * half)) & 0xffffu;
+                uint32_t o[4];
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    // 4 bits -> 4 byte LSBs: bit i lands on bit 8i, no carries
+                    const uint32_t sb = (((sh >> (4 * q)) & 15u) * 0x204081u) & 0x01010101u;
+                    const uint32_t nb = (((nh >> (4 * q)) & 15u) * 0x204081u) & 0x01010101u;
+                    o[q] = nb | (sb * 0xffu);
+                }
+                frag[half * 32 + r] = make_uint4(o[0], o[1], o[2], o[3]);
+            }
         }
     }
 }
@@ -426,6 +439,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
 #pragma unroll
     for (int j = 0; j < NB; j++) arrive(f[j], std::integral_constant<int, 0>{});
 
+    // ternary hand-over: whether every lane of a pixel block may take the compare-free form
+    bool direct_q[2] = {false, false};
+    if constexpr (QMODE == 1) {
+#pragma unroll
+        for (int b = 0; b < 2; b++) direct_q[b] = __all(tern_direct_applies(alpha, qthr[b])) != 0;
+    }
     // Block id = 2*a + b; wavefront ks of a tile finishes the blocks with id % S == ks and hands
     // the others over through LDS.  Every copy below names its accumulator registers statically,
     // under a wave-uniform branch, so that no register array is indexed at run time.
@@ -477,15 +496,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
             const uint32_t qc = (uint32_t)min(q, M - 1);
             const uint32_t img = fastdiv(qc, dOHW);
             const uint32_t pix = qc - img * (uint32_t)OHW;
-            // r = acc - bias: both are integers below 2^24 in fp32, and so is their difference
+            // r = acc - bias: both are integers below 2^24 in fp32, and so is their difference (only BNN has a bias)
             const float fbias = (float)bias;
+            const bool direct = QMODE == 1 && direct_q[b];   // wave-uniform
             float vals[16];
+            if (!direct) {
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const float fr = mine[e] - fbias;
-                // form 0: scale when f <= 0 (a zero becomes 0 * alpha); form 1: scale when r < 0
-                const bool scale = FORM0 ? (fr <= 0.0f) : (fr < 0.0f);
-                vals[e] = scale ? fr * alpha : fr;
+                for (int e = 0; e < 16; e++) {
+                    const float fr = FORM0 ? mine[e] : mine[e] - fbias;
+                    // form 0: scale when f <= 0 (a zero becomes 0 * alpha); form 1: scale when r < 0
+                    const bool scale = FORM0 ? (fr <= 0.0f) : (fr < 0.0f);
+                    vals[e] = scale ? fr * alpha : fr;
+                }
             }
             if constexpr (QMODE == 0) {
                 float* yq = Y + ((size_t)img * KN + kn0 + 32 * a + 4 * h) * OHW + pix;
@@ -509,7 +531,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
                 const float t = qthr[b];
                 constexpr bool tern = QMODE == 1;
                 uint32_t half[4];
-                if (kn0 + 32 * a + 32 <= KN) {   // uniform: the whole block holds real kernels
+                if (direct) {
+                    // ordinary slope and threshold: no compares, two nibbles per conversion (see tern_value_direct)
+                    const float t_big = t * 0x1p60f;
+                    float z[16];
+#pragma unroll
+                    for (int e = 0; e < 16; e++)
+                        z[e] = tern_value_direct(FORM0 ? mine[e] : mine[e] - fbias, alpha, t_big);
+                    if (kn0 + 32 * a + 32 > KN) {   // uniform: kernels past KN hold the padding lane
+#pragma unroll
+                        for (int e = 0; e < 16; e++)
+                            z[e] = kn0 + 32 * a + 8 * (e >> 2) + 4 * h + (e & 3) < KN ? z[e] : 0.0f;
+                    }
+                    const uint32_t d0 = pack_fp4x8(z[0], z[1], z[2], z[3], z[4], z[5], z[6], z[7]);
+                    const uint32_t d1 = pack_fp4x8(z[8], z[9], z[10], z[11], z[12], z[13], z[14], z[15]);
+                    half[0] = d0 & 0xffffu;
+                    half[1] = d0 >> 16;
+                    half[2] = d1 & 0xffffu;
+                    half[3] = d1 >> 16;
+                } else if (kn0 + 32 * a + 32 <= KN) {   // uniform: the whole block holds real kernels
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
                         half[g] = 0u;
@@ -581,7 +621,7 @@ hipError_t launch_gemm(const uint4* Pf, const uint4* Qf, float* Y, int M, int KN
 
 template <bool F4>
 hipError_t launch_expand(bool tern, const uint32_t* rows_ptr, int rows, int G, uint4* out, hipStream_t st) {
-    dim3 grid((rows + 31) / 32, G);
+    dim3 grid((rows + 31) / 32, (G + 3) / 4);   // 4 groups per workgroup (kGPB in the kernel)
     if (grid.y > 65535) return hipErrorInvalidValue;
     if (tern) hipLaunchKernelGGL((k_expand<F4, true>), grid, dim3(256), 0, st, rows_ptr, rows, G, out);
     else hipLaunchKernelGGL((k_expand<F4, false>), grid, dim3(256), 0, st, rows_ptr, rows, G, out);

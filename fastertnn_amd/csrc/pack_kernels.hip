@@ -382,6 +382,69 @@ __global__ __launch_bounds__(256) void k_dense_rows_f4(const uint32_t* __restric
     }
 }
 
+// The same with the kernel window known at compile time (the 3x3 and 7x7 windows of first layers): the tap of
+// every word position is then a constant, so the row and column of a tap are looked up in per-thread tables
+// filled once (clamped index, validity), its address is one add, and it enters the word with one or two
+// shift-or instructions.
+template <bool TERN, int C, int KH, int KW>
+__global__ __launch_bounds__(256) void k_dense_rows_f4_win(const uint32_t* __restrict__ Pq, int H, int W, int OHW,
+                                                           int OW, int H_pad, int W_pad, int H_stride, int W_stride,
+                                                           FastDiv dOW, uint4* __restrict__ A4) {
+    constexpr int T = 64 / C, taps = KH * KW, Kd = (taps + T - 1) / T;
+    constexpr uint32_t padv = TERN ? 0u : 0x22222222u;
+    constexpr uint32_t cmask = C >= 8 ? 0xffffffffu : ((1u << (4 * (C & 7))) - 1u);
+    const int pix = blockIdx.x * 256 + threadIdx.x, n = blockIdx.y;
+    if (pix >= OHW) return;
+    const int oh = (int)fastdiv((uint32_t)pix, dOW), ow = pix - oh * OW;
+    const int ih0 = oh * H_stride - H_pad, iw0 = ow * W_stride - W_pad;
+    const uint32_t* img = Pq + (size_t)n * H * W;
+    int rowoff[KH], col[KW];
+    bool rowok[KH], colok[KW];
+#pragma unroll
+    for (int kh = 0; kh < KH; kh++) {
+        const int ih = ih0 + kh;
+        rowok[kh] = (unsigned)ih < (unsigned)H;
+        rowoff[kh] = (rowok[kh] ? ih : 0) * W;
+    }
+#pragma unroll
+    for (int kw = 0; kw < KW; kw++) {
+        const int iw = iw0 + kw;
+        colok[kw] = (unsigned)iw < (unsigned)W;
+        col[kw] = colok[kw] ? iw : 0;
+    }
+#pragma unroll
+    for (int d = 0; d < Kd; d++) {
+        uint32_t o[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) o[i] = 0u;
+#pragma unroll
+        for (int j = 0; j < T; j++) {
+            const int tap = d * T + j;
+            const int bit = 4 * j * C, lo = bit >> 5, sh = bit & 31;
+            uint32_t v;
+            if (tap < taps) {   // compile-time after unrolling
+                const int kh = tap / KW, kw = tap % KW;
+                const uint32_t raw = img[rowoff[kh] + col[kw]];
+                v = ((rowok[kh] && colok[kw]) ? raw : padv) & cmask;
+            } else {
+                v = padv & cmask;
+            }
+            o[lo] |= v << sh;
+            if (sh + 4 * C > 32) o[lo + 1] |= v >> (32 - sh);
+        }
+        // lanes past T * C hold the padding lane of the type
+        constexpr int used = 4 * T * C;   // bits
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if (32 * i >= used) o[i] |= padv;
+            else if (32 * (i + 1) > used) o[i] |= padv & ~((1u << (used - 32 * i)) - 1u);
+        }
+        uint4* dst = A4 + (((size_t)n * Kd + d) * OHW + pix) * 2;
+        dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
+        dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
+    }
+}
+
 // weights: one work-item per (kernel, dense word); source rows are the reference's packed rows
 // with C_pack = 1 (word index = tap)
 template <bool TERN>
@@ -465,20 +528,26 @@ hipError_t launch_dense_rows_f4(bool ternary, const float* d_x, const float* d_t
     (void)T;
     if (ternary) hipLaunchKernelGGL((k_quantize_nib<true>), gq, dim3(256), 0, st, d_x, d_thr, C, HW, Pq);
     else hipLaunchKernelGGL((k_quantize_nib<false>), gq, dim3(256), 0, st, d_x, d_thr, C, HW, Pq);
+#define FTNN_DENSE_WIN(TERN_, C_, K_)                                                                             \
+    hipLaunchKernelGGL((k_dense_rows_f4_win<TERN_, C_, K_, K_>), gr, dim3(256), 0, st, Pq, H, W, OHW, OW, H_pad, W_pad, \
+                       H_stride, W_stride, dOW, A4)
+#define FTNN_DENSE_T(TERN_, C_)                                                                                     \
+    if (kH == 3 && kW == 3) FTNN_DENSE_WIN(TERN_, C_, 3);                                                           \
+    else if (kH == 7 && kW == 7) FTNN_DENSE_WIN(TERN_, C_, 7);                                                      \
+    else hipLaunchKernelGGL((k_dense_rows_f4<TERN_, C_>), gr, dim3(256), 0, st, Pq, H, W, OHW, OW, kW, kH * kW, Kd,    \
+                            H_pad, W_pad, H_stride, W_stride, dOW, A4)
 #define FTNN_DENSE(C_)                                                                                              \
     case C_:                                                                                                        \
-        if (ternary)                                                                                                \
-            hipLaunchKernelGGL((k_dense_rows_f4<true, C_>), gr, dim3(256), 0, st, Pq, H, W, OHW, OW, kW, kH * kW, Kd,  \
-                               H_pad, W_pad, H_stride, W_stride, dOW, A4);                                          \
-        else                                                                                                        \
-            hipLaunchKernelGGL((k_dense_rows_f4<false, C_>), gr, dim3(256), 0, st, Pq, H, W, OHW, OW, kW, kH * kW, Kd, \
-                               H_pad, W_pad, H_stride, W_stride, dOW, A4);                                          \
+        if (ternary) { FTNN_DENSE_T(true, C_); }                                                                    \
+        else { FTNN_DENSE_T(false, C_); }                                                                           \
         break;
     switch (C) {
         FTNN_DENSE(1) FTNN_DENSE(2) FTNN_DENSE(3) FTNN_DENSE(4) FTNN_DENSE(5) FTNN_DENSE(6) FTNN_DENSE(7) FTNN_DENSE(8)
         default: return hipErrorInvalidValue;
     }
 #undef FTNN_DENSE
+#undef FTNN_DENSE_T
+#undef FTNN_DENSE_WIN
     return hipGetLastError();
 }
 

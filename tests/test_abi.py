@@ -152,3 +152,11 @@ def test_build_refuses_scratch_in_hand_counted_kernels():
         build.check_no_scratch("mfma_kernels.hip", ok.replace("lane]: 0", "lane]: 60"))
     with pytest.raises(RuntimeError, match="no resource remarks"):
         build.check_no_scratch("mfma_kernels.hip", "")
+
+
+def test_popcount_probe_is_built_beside_the_library():
+    """bench.py runs it as a child process for the measured vector-ALU issue rate"""
+    import os
+    from fastertnn_amd import build
+    assert os.path.exists(build.LIB)
+    assert os.access(build.PROBE, os.X_OK)
