@@ -88,6 +88,19 @@ __device__ __forceinline__ uint32_t pack_fp4x8(float z0, float z1, float z2, flo
     return d;
 }
 
+// Hand-over store of one 32-kernel block: lanes l and l ^ 32 hold the nibbles of one pixel, lane half h those of
+// kernels 8 q + 4 h + {0..3}, as d0 (q = 0, 1) and d1 (q = 2, 3), 16 bits per q.  Returns the 8 bytes lane h
+// stores at byte 8 h of the block's 16: kernels in order.  v_permlane32_swap exchanges the upper half of d0 with the
+// lower half of d1, after which both lane halves combine their pair the same way.
+__device__ __forceinline__ uint2 exchange_halves(uint32_t d0, uint32_t d1) {
+    const auto r = __builtin_amdgcn_permlane32_swap(d0, d1, false, false);
+    // lanes 0..31: r[0] = own d0, r[1] = d0 of lane + 32; lanes 32..63: r[0] = d1 of lane - 32, r[1] = own d1
+    uint2 out;
+    out.x = (r[0] & 0xffffu) | (r[1] << 16);
+    out.y = (r[0] >> 16) | (r[1] & 0xffff0000u);
+    return out;
+}
+
 // record a failure text for ftnn_last_error(); returns `code`
 int fail(int code, const char* fmt, ...);
 

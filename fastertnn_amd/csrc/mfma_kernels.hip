@@ -545,7 +545,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
                     }
                     const uint32_t d0 = pack_fp4x8(z[0], z[1], z[2], z[3], z[4], z[5], z[6], z[7]);
                     const uint32_t d1 = pack_fp4x8(z[8], z[9], z[10], z[11], z[12], z[13], z[14], z[15]);
-                    half[0] = d0 & 0xffffu;
+                    half[0] = d0 & 0xffffu;   // (split and re-joined below at no cost: the compiler folds it)
                     half[1] = d0 >> 16;
                     half[2] = d1 & 0xffffu;
                     half[3] = d1 >> 16;
@@ -566,16 +566,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
                                        << (4 * i);
                     }
                 }
-                const uint32_t send = h ? (half[0] | (half[1] << 16)) : (half[2] | (half[3] << 16));
-                const uint32_t recv = (uint32_t)__shfl_xor((int)send, 32, 64);
-                uint2 out;
-                if (h == 0) {
-                    out.x = half[0] | (recv << 16);
-                    out.y = half[1] | (recv & 0xffff0000u);
-                } else {
-                    out.x = (recv & 0xffffu) | (half[2] << 16);
-                    out.y = (recv >> 16) | (half[3] << 16);
-                }
+                const uint2 out = exchange_halves(half[0] | (half[1] << 16), half[2] | (half[3] << 16));
                 const size_t word = ((size_t)img * gridDim.y + blockIdx.y) * OHW + pix;
                 if (q < M) *reinterpret_cast<uint2*>(static_cast<unsigned char*>(qo.p4) + word * 32 + 16 * a + 8 * h) = out;
             }
