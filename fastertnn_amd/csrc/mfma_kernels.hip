@@ -574,6 +574,171 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
     });
 }
 
+// The same layer on tiles of 32 kernels x 32 pixels, for layers with few tiles of 64 x 64: a wavefront moves a
+// bounded number of bytes per cycle from a cold L2 whatever its prefetch depth (600-700 cycles per K word of a
+// 64 x 64 tile, measured), so a small layer gets faster only with more wavefronts, on more compute units.  A
+// workgroup is one tile; its four wavefronts split the K loop four ways (word w to wavefront w % 4, one weight and
+// one activation fragment per word), wavefronts 1..3 hand their partial block over through LDS and wavefront 0
+// finishes it.  Kernel tiles come in pairs under the hand-over (a pixel's 64-channel word is written by two
+// workgroups, 16 bytes each; a tile past KN writes padding lanes).
+template <bool ABIN, bool FORM0, int QMODE>
+__global__ __launch_bounds__(256) void k_conv_f4_small(const uint4* __restrict__ P4, const uint4* __restrict__ Wf,
+                                                       float* __restrict__ Y, int M, int KN, int OHW, int KB, int bias,
+                                                       float alpha, FastDiv dOHW, ConvGeom cg, QuantOut qo) {
+    constexpr int S = 4, NB = 3;
+    __shared__ float4 red[3 * 4 * 64];   // [wavefront - 1][e / 4][lane]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int ks = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int h = lane >> 5, lr = lane & 31;
+    const int px0 = blockIdx.x * 32, kn0 = blockIdx.y * 32;
+
+    const int q = px0 + lr;
+    const uint32_t qc = (uint32_t)min(q, M - 1);
+    const uint32_t img = fastdiv(qc, dOHW);
+    const uint32_t pix = qc - img * (uint32_t)OHW;
+    const int oh = (int)fastdiv(pix, cg.dOW), ow = (int)pix - oh * cg.OW;
+    const int ih0 = oh * cg.H_stride - cg.H_pad, iw0 = ow * cg.W_stride - cg.W_pad;
+    const uint32_t pb = img * (uint32_t)(cg.CP * cg.H * cg.W);   // image of P4[n][C_pack][pixel]
+    float qthr = 0.0f;
+    if constexpr (QMODE != 0) qthr = qo.thr[img];   // fetched ahead of the hand-counted loads (see k_conv_f4)
+    const int HWin = cg.H * cg.W;
+    const int rbmax = (KN + 31) / 32 - 1;
+    const uint4* wb = Wf + (size_t)min(kn0 / 32, rbmax) * KB * 64 + lane;
+
+    v16f acc;
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+    const uint32_t fillv = ABIN ? 0x22222222u : 0u;
+
+    struct Frag {
+        v4i w, x;
+        bool in;
+    };
+    auto ld16 = [](v4i& dst, const uint4* src) {
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(dst) : "v"(src) : "memory");
+    };
+    auto load = [&](int w, Frag& f) {   // w is wave-uniform
+        const int tap = (int)fastdiv((uint32_t)w, cg.dCP), ic = w - tap * cg.CP;
+        const int kh = (int)fastdiv((uint32_t)tap, cg.dKW), kw = tap - kh * cg.KW;
+        ld16(f.w, wb + (size_t)w * 64);
+        const int ih = ih0 + kh, iw = iw0 + kw;
+        f.in = (unsigned)ih < (unsigned)cg.H && (unsigned)iw < (unsigned)cg.W;
+        const size_t o = (size_t)(pb + (uint32_t)(ic * HWin + (f.in ? ih * cg.W + iw : 0))) * 2 + h;
+        ld16(f.x, P4 + o);
+    };
+    auto arrive = [](Frag& f, auto outstanding) {
+        asm volatile("s_waitcnt vmcnt(%2)" : "+v"(f.w), "+v"(f.x) : "n"(decltype(outstanding)::value) : "memory");
+    };
+    auto compute = [&](const Frag& f) {
+        v8i x, wv;
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] = f.in ? f.x[i] : (int)fillv;
+#pragma unroll
+        for (int i = 4; i < 8; i++) x[i] = 0;
+        wv = v8i{f.w[0], f.w[1], f.w[2], f.w[3], 0, 0, 0, 0};
+        acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wv, x, acc, 4, 4, 0, 0, 0, 0);
+    };
+
+    // as in k_conv_f4: register sets rotate by name, loads past the last word re-read it and are not multiplied
+    const int K = cg.K;
+    Frag f[NB];
+    std::integral_constant<int, 2 * (NB - 1)> ahead;
+    int w = ks;
+#pragma unroll
+    for (int j = 0; j < NB - 1; j++) load(min(w + S * j, K - 1), f[j]);
+    for (; w < K; w += S * NB) {
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+            load(min(w + S * (j + NB - 1), K - 1), f[(j + NB - 1) % NB]);
+            arrive(f[j], ahead);
+            if (j == 0 || w + S * j < K) compute(f[j]);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < NB; j++) arrive(f[j], std::integral_constant<int, 0>{});
+
+    if (ks != 0) {
+        float4* dst = red + (size_t)((ks - 1) * 4) * 64 + lane;
+#pragma unroll
+        for (int e4 = 0; e4 < 4; e4++)
+            dst[e4 * 64] = make_float4(acc[4 * e4], acc[4 * e4 + 1], acc[4 * e4 + 2], acc[4 * e4 + 3]);
+    }
+    __syncthreads();
+    if (ks != 0) return;
+#pragma unroll
+    for (int v = 0; v < 3; v++) {
+        const float4* src = red + (size_t)(v * 4) * 64 + lane;
+#pragma unroll
+        for (int e4 = 0; e4 < 4; e4++) {
+            const float4 t = src[e4 * 64];
+            acc[4 * e4] += t.x;
+            acc[4 * e4 + 1] += t.y;
+            acc[4 * e4 + 2] += t.z;
+            acc[4 * e4 + 3] += t.w;
+        }
+    }
+
+    // accumulator e: kernel = kn0 + 8*(e/4) + 4*h + e%4, pixel = px0 + lr
+    const float fbias = (float)bias;
+    const bool whole = kn0 + 32 <= KN;   // uniform
+    const bool direct = QMODE == 1 && __all(tern_direct_applies(alpha, qthr)) != 0;
+    float vals[16];
+    if (!direct) {
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const float fr = FORM0 ? acc[e] : acc[e] - fbias;
+            const bool scale = FORM0 ? (fr <= 0.0f) : (fr < 0.0f);
+            vals[e] = scale ? fr * alpha : fr;
+        }
+    }
+    if constexpr (QMODE == 0) {
+        float* yq = Y + ((size_t)img * KN + kn0 + 4 * h) * OHW + pix;
+        if (q < M) {
+            if (whole) {
+#pragma unroll
+                for (int e = 0; e < 16; e++) yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = vals[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const int p = kn0 + 8 * (e >> 2) + 4 * h + (e & 3);
+                    if (p < KN) yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = vals[e];
+                }
+            }
+        }
+    } else {
+        constexpr bool tern = QMODE == 1;
+        uint32_t d0, d1;
+        if (direct) {
+            const float t_big = qthr * 0x1p60f;
+            float z[16];
+#pragma unroll
+            for (int e = 0; e < 16; e++) z[e] = tern_value_direct(FORM0 ? acc[e] : acc[e] - fbias, alpha, t_big);
+            if (!whole) {
+#pragma unroll
+                for (int e = 0; e < 16; e++) z[e] = kn0 + 8 * (e >> 2) + 4 * h + (e & 3) < KN ? z[e] : 0.0f;
+            }
+            d0 = pack_fp4x8(z[0], z[1], z[2], z[3], z[4], z[5], z[6], z[7]);
+            d1 = pack_fp4x8(z[8], z[9], z[10], z[11], z[12], z[13], z[14], z[15]);
+        } else {
+            uint32_t half[4];
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                half[g] = 0u;
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    half[g] |= quant_nibble(vals[4 * g + i], qthr, tern, whole || kn0 + 8 * g + 4 * h + i < KN) << (4 * i);
+            }
+            d0 = half[0] | (half[1] << 16);
+            d1 = half[2] | (half[3] << 16);
+        }
+        const uint2 out = exchange_halves(d0, d1);
+        // this tile is half a 64-channel word: bytes 16 * (tile parity) of the pixel's 32
+        const size_t word = ((size_t)img * (gridDim.y >> 1) + (blockIdx.y >> 1)) * OHW + pix;
+        if (q < M)
+            *reinterpret_cast<uint2*>(static_cast<unsigned char*>(qo.p4) + word * 32 + 16 * (blockIdx.y & 1) + 8 * h) = out;
+    }
+}
+
 // tiles of 256 x 256 below which the 128 x 128 kernel is used (FTNN_MFMA_SMALL_BELOW: tuning aid)
 inline int64_t mfma_small_tile_below() {
     static const int64_t v = []() {
@@ -663,10 +828,16 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
     // alone do that (a tile = 64 kernels x 64 pixels)
     const int64_t tiles = ((M + 63) / 64) * ((KN + 63) / 64);
     int split = tiles >= 600 ? 1 : (tiles >= 450 ? 2 : 4);   // measured on MI355X (1024 SIMDs)
+    static const int min_words = getenv("FTNN_CONV_SPLIT_MIN_WORDS") ? atoi(getenv("FTNN_CONV_SPLIT_MIN_WORDS")) : 1;
+    while (split > 1 && cg.K < min_words * split) split /= 2;   // no wavefront without K words of its own
     static const char* tune = getenv("FTNN_CONV_SPLIT");   // tuning aid: force the K split
     if (tune) split = atoi(tune);
     const int wpb = 4, tpb = wpb / split;   // wavefronts and pixel tiles per workgroup (see the kernel)
+    // few 64 x 64 tiles: tiles of 32 x 32, four times the workgroups (k_conv_f4_small)
+    static const int small_below = getenv("FTNN_CONV_SMALL_BELOW") ? atoi(getenv("FTNN_CONV_SMALL_BELOW")) : 150;
+    const bool small = tiles < small_below;
     dim3 grid((unsigned)(((M + 63) / 64 + tpb - 1) / tpb), (unsigned)((KN + 63) / 64));
+    if (small) grid = dim3((unsigned)((M + 31) / 32), (unsigned)(qo.mode != 0 ? 2 * ((KN + 63) / 64) : (KN + 31) / 32));
     if (M > 0x7fffff00LL || grid.y > 65535) return hipErrorInvalidValue;   // pixel indices stay below 2^31
     const uint4* P4 = static_cast<const uint4*>(d_p4);
     const uint4* Wf = static_cast<const uint4*>(d_wf);
@@ -689,6 +860,7 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
     auto by_split = [&](auto abin, auto form0, auto qmode) -> hipError_t {
         constexpr bool A = decltype(abin)::value, F = decltype(form0)::value;
         constexpr int Q = decltype(qmode)::value;
+        if (small) return launch(std::integral_constant<decltype(&k_conv_f4_small<A, F, Q>), &k_conv_f4_small<A, F, Q>>{});
         // three register sets: deeper prefetch measured no faster at any layer size
         if (split == 1) return launch(std::integral_constant<decltype(&k_conv_f4<A, F, Q, 1, 3>), &k_conv_f4<A, F, Q, 1, 3>>{});
         if (split == 2) return launch(std::integral_constant<decltype(&k_conv_f4<A, F, Q, 2, 3>), &k_conv_f4<A, F, Q, 2, 3>>{});

@@ -299,9 +299,9 @@ class Net:
         return out
 
     def close(self):
-        if self._h:
+        if self._h and _L is not None:   # at interpreter shutdown the module's globals may be gone already
             _L.ftnn_net_destroy(self._h)
-            self._h = None
+        self._h = None
 
     def __del__(self):
         self.close()
