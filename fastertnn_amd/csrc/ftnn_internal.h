@@ -77,6 +77,41 @@ __device__ __forceinline__ float tern_value_direct(float r, float alpha, float t
     const float neg = __builtin_amdgcn_fmed3f(__builtin_fmaf(r * alpha, -0x1p60f, -t_big), 0.0f, 1.0f);
     return pos - neg;
 }
+// The binary hand-over the same way: the bit is PReLU(r) < t.  For t > 0 that is r < t (r <= 0 gives PReLU <= 0 < t),
+// for t <= 0 it is r * alpha < t (r >= 0 gives PReLU >= 0 >= t).  With alpha = 0 or 2^-20 <= alpha <= 2^20 and t = 0
+// or 2^-20 <= |t| <= 2^40 a positive difference t - v is at least 2^-44; the result is -1 (bit set) or +1 as a float.
+// `t_pos` must be the same for all lanes of the wavefront.
+__device__ __forceinline__ bool bin_direct_applies(float alpha, float t) {
+    const float at = __builtin_fabsf(t);
+    return (alpha == 0.0f || (alpha >= 0x1p-20f && alpha <= 0x1p20f)) && (t == 0.0f || (at >= 0x1p-20f && at <= 0x1p40f));
+}
+__device__ __forceinline__ float bin_value_direct(float r, float alpha, float t_big /* t * 2^60 */, bool t_pos) {
+    const float v = t_pos ? r : r * alpha;
+    const float below = __builtin_amdgcn_fmed3f(__builtin_fmaf(v, -0x1p60f, t_big), 0.0f, 1.0f);
+    return __builtin_fmaf(below, -2.0f, 1.0f);
+}
+// Both hand-overs behind one face: whether the wavefront may take the compare-free form for its thresholds
+// (mode 1 ternary, 2 binary; for binary all thresholds must lie on the same side of zero), and the value.
+struct DirectQuant {
+    bool ok, t_pos;
+};
+template <int QMODE>
+__device__ __forceinline__ DirectQuant direct_quant(float alpha, float t) {
+    DirectQuant d = {false, false};
+    if constexpr (QMODE == 1) {
+        d.ok = __all(tern_direct_applies(alpha, t)) != 0;
+    } else if constexpr (QMODE == 2) {
+        const bool fits = bin_direct_applies(alpha, t);
+        d.t_pos = __all(fits && t > 0.0f) != 0;
+        d.ok = d.t_pos || __all(fits && !(t > 0.0f)) != 0;
+    }
+    return d;
+}
+template <int QMODE>
+__device__ __forceinline__ float direct_value(float r, float alpha, float t_big, bool t_pos, bool live) {
+    if constexpr (QMODE == 1) return live ? tern_value_direct(r, alpha, t_big) : 0.0f;
+    else return live ? bin_value_direct(r, alpha, t_big, t_pos) : 1.0f;   // padding lanes: 0 / +1
+}
 // eight values out of {+1, -1, +0} -> one dword of E2M1 nibbles, value k in nibble k
 __device__ __forceinline__ uint32_t pack_fp4x8(float z0, float z1, float z2, float z3, float z4, float z5, float z6,
                                                float z7) {

@@ -439,11 +439,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
 #pragma unroll
     for (int j = 0; j < NB; j++) arrive(f[j], std::integral_constant<int, 0>{});
 
-    // ternary hand-over: whether every lane of a pixel block may take the compare-free form
-    bool direct_q[2] = {false, false};
-    if constexpr (QMODE == 1) {
+    // hand-over: whether every lane of a pixel block may take the compare-free form
+    DirectQuant direct_q[2] = {{false, false}, {false, false}};
+    if constexpr (QMODE != 0) {
 #pragma unroll
-        for (int b = 0; b < 2; b++) direct_q[b] = __all(tern_direct_applies(alpha, qthr[b])) != 0;
+        for (int b = 0; b < 2; b++) direct_q[b] = direct_quant<QMODE>(alpha, qthr[b]);
     }
     // Block id = 2*a + b; wavefront ks of a tile finishes the blocks with id % S == ks and hands
     // the others over through LDS.  Every copy below names its accumulator registers statically,
@@ -498,7 +498,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
             const uint32_t pix = qc - img * (uint32_t)OHW;
             // r = acc - bias: both are integers below 2^24 in fp32, and so is their difference (only BNN has a bias)
             const float fbias = (float)bias;
-            const bool direct = QMODE == 1 && direct_q[b];   // wave-uniform
+            const bool direct = QMODE != 0 && direct_q[b].ok;   // wave-uniform
             float vals[16];
             if (!direct) {
 #pragma unroll
@@ -534,14 +534,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
                 if (direct) {
                     // ordinary slope and threshold: no compares, two nibbles per conversion (see tern_value_direct)
                     const float t_big = t * 0x1p60f;
+                    const bool t_pos = direct_q[b].t_pos;
                     float z[16];
-#pragma unroll
-                    for (int e = 0; e < 16; e++)
-                        z[e] = tern_value_direct(FORM0 ? mine[e] : mine[e] - fbias, alpha, t_big);
-                    if (kn0 + 32 * a + 32 > KN) {   // uniform: kernels past KN hold the padding lane
+                    if (kn0 + 32 * a + 32 <= KN) {   // uniform: the whole block holds real kernels
 #pragma unroll
                         for (int e = 0; e < 16; e++)
-                            z[e] = kn0 + 32 * a + 8 * (e >> 2) + 4 * h + (e & 3) < KN ? z[e] : 0.0f;
+                            z[e] = direct_value<QMODE>(FORM0 ? mine[e] : mine[e] - fbias, alpha, t_big, t_pos, true);
+                    } else {   // kernels past KN hold the padding lane
+#pragma unroll
+                        for (int e = 0; e < 16; e++)
+                            z[e] = direct_value<QMODE>(FORM0 ? mine[e] : mine[e] - fbias, alpha, t_big, t_pos,
+                                                       kn0 + 32 * a + 8 * (e >> 2) + 4 * h + (e & 3) < KN);
                     }
                     const uint32_t d0 = pack_fp4x8(z[0], z[1], z[2], z[3], z[4], z[5], z[6], z[7]);
                     const uint32_t d1 = pack_fp4x8(z[8], z[9], z[10], z[11], z[12], z[13], z[14], z[15]);
@@ -681,7 +684,8 @@ __global__ __launch_bounds__(256) void k_conv_f4_small(const uint4* __restrict__
     // accumulator e: kernel = kn0 + 8*(e/4) + 4*h + e%4, pixel = px0 + lr
     const float fbias = (float)bias;
     const bool whole = kn0 + 32 <= KN;   // uniform
-    const bool direct = QMODE == 1 && __all(tern_direct_applies(alpha, qthr)) != 0;
+    const DirectQuant dq = direct_quant<QMODE>(alpha, qthr);
+    const bool direct = QMODE != 0 && dq.ok;
     float vals[16];
     if (!direct) {
 #pragma unroll
@@ -712,10 +716,12 @@ __global__ __launch_bounds__(256) void k_conv_f4_small(const uint4* __restrict__
             const float t_big = qthr * 0x1p60f;
             float z[16];
 #pragma unroll
-            for (int e = 0; e < 16; e++) z[e] = tern_value_direct(FORM0 ? acc[e] : acc[e] - fbias, alpha, t_big);
-            if (!whole) {
+            for (int e = 0; e < 16; e++)
+                z[e] = direct_value<QMODE>(FORM0 ? acc[e] : acc[e] - fbias, alpha, t_big, dq.t_pos, true);
+            if (!whole) {   // kernels past KN: the padding lane
 #pragma unroll
-                for (int e = 0; e < 16; e++) z[e] = kn0 + 8 * (e >> 2) + 4 * h + (e & 3) < KN ? z[e] : 0.0f;
+                for (int e = 0; e < 16; e++)
+                    z[e] = kn0 + 8 * (e >> 2) + 4 * h + (e & 3) < KN ? z[e] : (QMODE == 1 ? 0.0f : 1.0f);
             }
             d0 = pack_fp4x8(z[0], z[1], z[2], z[3], z[4], z[5], z[6], z[7]);
             d1 = pack_fp4x8(z[8], z[9], z[10], z[11], z[12], z[13], z[14], z[15]);

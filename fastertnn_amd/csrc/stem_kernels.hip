@@ -37,9 +37,9 @@ struct StemGeom {
 
 // ABIN / FORM0 / QMODE as in k_conv_f4; C is compile-time so that every shift below is a constant.
 template <bool ABIN, bool FORM0, int QMODE, int C>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) void k_stem_f4(const float* __restrict__ x, const float* __restrict__ thr,
-                                                 const uint4* __restrict__ Wf, float* __restrict__ Y, int KN,
-                                                 int KB, int bias, float alpha, StemGeom g, QuantOut qo) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) void k_stem_f4(
+    const float* __restrict__ x, const float* __restrict__ thr, const uint4* __restrict__ Wf, float* __restrict__ Y,
+    int KN, int KB, int bias, float alpha, StemGeom g, QuantOut qo) {
     constexpr int T = 64 / C;                    // taps per word
     constexpr int J1 = 32 / C;                   // first tap that reaches into the upper half of a word
     constexpr int NI0 = (32 + C - 1) / C;        // taps that touch the lower half
@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
     constexpr uint32_t cmask = C >= 8 ? 0xffffffffu : ((1u << (4 * (C & 7))) - 1u);
     static_assert(4 * C * NI <= 160, "five dwords hold the taps of one half");
 
-    extern __shared__ uint32_t lds[];
+    extern __shared__ __align__(16) uint32_t lds[];
     const int PP = g.PH * g.PW;
     uint32_t* patch = lds;                 // [0, PP): the quantised patch; [PP, 2 PP): padding nibbles
     uint32_t* toff = lds + 2 * PP;         // [Kd][TT]: byte offset of a tap in the patch (or into the padding)
@@ -204,8 +204,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
     const float fbias = (float)bias;
     float qthr = 0.0f;
     if constexpr (QMODE != 0) qthr = qo.thr[n];
-    // ternary hand-over with an ordinary slope and threshold: the nibbles come straight from the accumulators
-    const bool direct = QMODE == 1 && tern_direct_applies(alpha, qthr);
+    // hand-over with an ordinary slope and threshold: the nibbles come straight from the accumulators
+    const DirectQuant dq = direct_quant<QMODE>(alpha, qthr);
+    const bool direct = QMODE != 0 && dq.ok;
     const float qthr_big = qthr * 0x1p60f;
 #pragma unroll
     for (int a = 0; a < 2; a++)
@@ -215,7 +216,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
             const int pix = live ? oh[b] * g.OW + ow[b] : 0;
             const bool whole = kn0 + 32 * a + 32 <= KN;   // uniform: the block holds real kernels only
             float vals[16];
-            if (QMODE != 1 || !direct) {
+            if (!direct) {
 #pragma unroll
                 for (int e = 0; e < 16; e++) {
                     const float fr = FORM0 ? acc[a][b][e] : acc[a][b][e] - fbias;   // only BNN has a bias
@@ -241,15 +242,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
                 // the same exchange as in k_conv_f4: lane h ends up with bytes 16 a + 8 h .. + 8 of the pixel's word
                 constexpr bool tern = QMODE == 1;
                 uint32_t half[4];
-                if (QMODE == 1 && direct) {
+                if (direct) {
                     float z[16];
-#pragma unroll
-                    for (int e = 0; e < 16; e++)
-                        z[e] = tern_value_direct(FORM0 ? acc[a][b][e] : acc[a][b][e] - fbias, alpha, qthr_big);
-                    if (!whole) {   // kernels past KN: the padding lane
+                    if (whole) {
 #pragma unroll
                         for (int e = 0; e < 16; e++)
-                            z[e] = kn0 + 32 * a + 8 * (e >> 2) + 4 * h + (e & 3) < KN ? z[e] : 0.0f;
+                            z[e] = direct_value<QMODE>(FORM0 ? acc[a][b][e] : acc[a][b][e] - fbias, alpha, qthr_big,
+                                                       dq.t_pos, true);
+                    } else {   // kernels past KN: the padding lane
+#pragma unroll
+                        for (int e = 0; e < 16; e++)
+                            z[e] = direct_value<QMODE>(FORM0 ? acc[a][b][e] : acc[a][b][e] - fbias, alpha, qthr_big,
+                                                       dq.t_pos, kn0 + 32 * a + 8 * (e >> 2) + 4 * h + (e & 3) < KN);
                     }
                     const uint32_t d0 = pack_fp4x8(z[0], z[1], z[2], z[3], z[4], z[5], z[6], z[7]);
                     const uint32_t d1 = pack_fp4x8(z[8], z[9], z[10], z[11], z[12], z[13], z[14], z[15]);

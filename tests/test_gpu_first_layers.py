@@ -52,14 +52,15 @@ def _chain(hip, oracle, batch, specs, x, seed):
 @pytest.mark.parametrize("c", range(1, 9))
 def test_first_layer_hand_over(hip, oracle, c):
     """a first layer followed by an fp4 layer of every activation kind: the ternary hand-over in its compare-free
-    form (ordinary slope and threshold) and in its select form (negative slope, negative or huge threshold, zero
-    slope), the binary hand-over; 70 kernels leave padding lanes in the second word"""
+    form (ordinary slope and threshold) and in its select form (negative slope, negative or huge threshold), the
+    binary hand-over in both forms as well (thresholds on either side of zero, tiny, huge); 70 kernels leave padding lanes in the second word"""
     batch = 2
     x = synth.normal(500 + c, (batch, c, 21, 26))
     first = (c, 21, 26, 70, 3, 3, 1, 1)
     second = (70, 21, 26, 40, 3, 3, 1, 2)
     cases = [(TNN, 0.5, 0.5), (TNN, 0.5, -0.5), (TNN, -1.0, 0.5), (TNN, 1e13, 0.5), (TNN, 0.0, 0.0), (TNN, 2.0, 0.25),
-             (TBN, 1.5, 1.0), (BTN, 0.5, 0.5), (BNN, -1.0, 0.25)]
+             (TBN, 1.5, 1.0), (BTN, 0.5, 0.5), (BNN, -1.0, 0.25), (BTN, 0.0, 0.5), (BTN, 1e-30, 0.5), (BNN, 1e13, 0.5),
+             (BTN, 0.25, -0.5), (BNN, -3.0, 0.0)]
     for first_typ in (TNN, BNN, TBN):
         for next_typ, next_thr, alpha in cases:
             print("case", c, TYPE_NAMES[first_typ], TYPE_NAMES[next_typ], next_thr, alpha, flush=True)
