@@ -271,19 +271,25 @@ RESNET18_LIKE = [  # (C, IH, IW, KN, KW, KH, pad, stride): stem, four stages wit
 ]
 
 
-def e2e_latency(torch, lib, batch, reps=10, cpu=True):
+def e2e_latency(torch, lib, batch, reps=10, cpu=True, typ=None):
     """the ResNet-18-like TNN stack chained on the device (eager launches and HIP-graph replay), and
     (cpu=True) the same chain through the reference's tnns_conv on one host core"""
     import numpy as np
-    from fastertnn_amd import TNN
+    from fastertnn_amd import TNN, act_is_ternary, weight_is_ternary
+    typ = TNN if typ is None else typ
+    at, wt = act_is_ternary(typ), weight_is_ternary(typ)
     g = torch.Generator(device="cuda")
     g.manual_seed(6)
     x = torch.randn((batch, 3, 224, 224), generator=g, device="cuda")
     layers = []
     for (c, ih, iw, kn, kw, kh, pad, stride) in RESNET18_LIKE:
-        w = torch.randint(-1, 2, (kn, c, kh, kw), generator=g, device="cuda", dtype=torch.int8).float()
-        qw = lib.pack_weights(w, torch.full((kn,), 0.5, device="cuda"), True)
-        layers.append(dict(type=TNN, shape=(c, ih, iw, kn, kw, kh, pad, stride), threshold=0.5, alpha=0.5, qw=qw))
+        if wt:
+            w = torch.randint(-1, 2, (kn, c, kh, kw), generator=g, device="cuda", dtype=torch.int8).float()
+        else:
+            w = torch.randint(0, 2, (kn, c, kh, kw), generator=g, device="cuda", dtype=torch.int8).float() * 2 - 1
+        qw = lib.pack_weights(w, torch.full((kn,), 0.5 if wt else 0.0, device="cuda"), wt)
+        layers.append(dict(type=typ, shape=(c, ih, iw, kn, kw, kh, pad, stride), threshold=0.5 if at else 0.0,
+                           alpha=0.5, qw=qw))
     net = lib.Net(batch, layers)
     y = torch.empty(net.out_shape, device="cuda")
     macs = sum(batch * lib.out_dim(ih, p, kh, s) * lib.out_dim(iw, p, kw, s) * kn * c * kh * kw
@@ -301,11 +307,11 @@ def e2e_latency(torch, lib, batch, reps=10, cpu=True):
     if cpu and O.Reference.available():
         ref = O.Reference()
         xh = x.cpu().numpy()
-        thr = np.full(batch, 0.5, np.float32)
+        thr = np.full(batch, 0.5 if at else 0.0, np.float32)
         t0 = time.perf_counter()
         for l in layers:
             c, ih, iw, kn, kw, kh, pad, stride = l["shape"]
-            xh = ref.conv(TNN, xh, thr, O.aligned_copy(l["qw"].cpu().numpy()), kn, kh, kw, pad, stride, 0.5)
+            xh = ref.conv(typ, xh, thr, O.aligned_copy(l["qw"].cpu().numpy()), kn, kh, kw, pad, stride, 0.5)
         out["cpu_ms"] = round((time.perf_counter() - t0) * 1e3, 1)
         out["bit_exact_vs_reference"] = bool(y.cpu().numpy().tobytes() == np.ascontiguousarray(xh).tobytes())
     net.close()
@@ -540,6 +546,8 @@ def main():
             "reference_gemm_sweep": reference_gemm_sweep(torch, lib),
             "reference_e2e_networks_b8": reference_networks(torch, lib),
             "tnn_resnet18_like_other_batches": {"b%d" % b: e2e_latency(torch, lib, b, cpu=False) for b in (1, 8, 128)},
+            "other_types_resnet18_like_b32": {n: e2e_latency(torch, lib, 32, cpu=False, typ=t)
+                                              for n, t in (("tbn", 1), ("btn", 2), ("bnn", 3))},
         }
 
     line = {
