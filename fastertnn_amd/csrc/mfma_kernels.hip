@@ -34,18 +34,19 @@ typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int kKF = 2;   // fragments per row-block and step
-constexpr int kNS = 4;   // LDS ring depth
+// Ring of NS LDS buffers, each holding KF fragments (K words for fp4) per row-block: one barrier per KF fragments.
 // A workgroup of 2 x 2 wavefronts computes (64 WT) x (64 WT) results, a wavefront WT x WT blocks of 32 x 32:
 // WT = 4 for problems with enough 256 x 256 tiles to fill the chip, WT = 2 (128 x 128) below that.
-template <int WT>
+template <int WT, int KF, int NS>
 struct Tile {
     static constexpr int RB = 2 * WT;             // row-blocks per operand side
-    static constexpr int FR = 2 * RB * kKF;       // fragments per step: (RB P + RB Q row-blocks) x kKF
+    static constexpr int FR = 2 * RB * KF;        // fragments per step: (RB P + RB Q row-blocks) x KF
     static constexpr int FW = FR / 4;             // fragments staged by one wavefront per step
     static constexpr int NL = 2 * WT;             // LDS reads per wavefront and k fragment
-    static constexpr size_t lds_bytes = (size_t)kNS * FR * 1024;
-    static_assert(FW == NL && (WT * WT) % NL == 0, "one staged fragment and WT/2 multiplies per LDS read");
+    static constexpr int DPI = FW / NL;           // fragments a wavefront stages per LDS read of the last fragment
+    static constexpr size_t lds_bytes = (size_t)NS * FR * 1024;
+    static_assert(FW % NL == 0 && (WT * WT) % NL == 0, "whole staged fragments and WT/2 multiplies per LDS read");
+    static_assert(NS >= 2 && KF % 2 == 0, "register sets alternate per fragment");
 };
 
 // ------------------------------------------------------------------ expansion
@@ -159,13 +160,14 @@ __device__ __forceinline__ void dma16(const uint4* gsrc, uint32_t lds_byte_addr)
 // The epilogue computes r = acc - bias, then PReLU in the reference's form for the type:
 // form 0 "f = r; if (f <= 0) f *= alpha" (mm_p2_final_tnn_avx2.c:204-208), form 1
 // "r >= 0 ? r : alpha * r" (mm_p2_final_tbn_avx2.c:73).
-template <bool F4, bool SWAP, int WT>
+template <bool F4, bool SWAP, int WT, int kKF, int kNS>
 __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, const uint4* __restrict__ Qf,
                                               float* __restrict__ Y, int M, int KN, int OHW, int KB,
                                               int bias, int form, float alpha) {
     extern __shared__ uint4 lds[];   // kNS buffers of kFR KiB
     typedef typename Acc<F4>::type acc_t;
-    constexpr int RB = Tile<WT>::RB, kFR = Tile<WT>::FR, kFW = Tile<WT>::FW, NL = Tile<WT>::NL;
+    typedef Tile<WT, kKF, kNS> TL;
+    constexpr int RB = TL::RB, kFR = TL::FR, kFW = TL::FW, NL = TL::NL, DPI = TL::DPI;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wy = wave >> 1, wx = wave & 1;
@@ -249,7 +251,11 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
                 const uint32_t dst = lds0 + (uint32_t)(s % kNS) * (kFR * 1024) + wave * (kFW * 1024);
 #pragma unroll
                 for (int i = 0; i < NL; i++) {
-                    if (FULL) dma16(src[i] + (size_t)(s + kNS) * kKF * 64, dst + i * 1024);
+                    if (FULL) {
+#pragma unroll
+                        for (int j = 0; j < DPI; j++)
+                            dma16(src[i * DPI + j] + (size_t)(s + kNS) * kKF * 64, dst + (i * DPI + j) * 1024);
+                    }
                     if (do_ld) ldone((s + 1) % kNS, 0, set ^ 1, i);
                     mfma2(set, i);
                     __builtin_amdgcn_sched_barrier(0);
@@ -754,11 +760,11 @@ inline int64_t mfma_small_tile_below() {
     return v;
 }
 
-template <bool F4, bool SWAP, int WT>
+template <bool F4, bool SWAP, int WT, int KF, int NS>
 hipError_t launch_gemm_tile(const uint4* Pf, const uint4* Qf, float* Y, int M, int KN, int OHW, int KB,
                             int bias, int form, float alpha, hipStream_t st) {
-    auto kern = k_mfma<F4, SWAP, WT>;
-    constexpr size_t lds_bytes = Tile<WT>::lds_bytes;
+    auto kern = k_mfma<F4, SWAP, WT, KF, NS>;
+    constexpr size_t lds_bytes = Tile<WT, KF, NS>::lds_bytes;
     // the opt-in to more than 64 KiB of dynamic LDS is per kernel; done once, thread-safe
     static const hipError_t configured = hipFuncSetAttribute(
         reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -777,8 +783,10 @@ hipError_t launch_gemm(const uint4* Pf, const uint4* Qf, float* Y, int M, int KN
     // 256 compute units; below that, 128 x 128 tiles (two workgroups fit a compute unit)
     const int64_t big = (((int64_t)M + 255) / 256) * ((KN + 255) / 256);
     bool small = big < mfma_small_tile_below();
-    return small ? launch_gemm_tile<F4, SWAP, 2>(Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha, st)
-                 : launch_gemm_tile<F4, SWAP, 4>(Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha, st);
+    // two fragments per step and a ring of four: four fragments per step with a ring of two (the same LDS, half
+    // the barriers) measured 0.87 against 0.76 ms on 8192 x 8192 x 32768 -- the ring then no longer covers the loads
+    return small ? launch_gemm_tile<F4, SWAP, 2, 2, 4>(Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha, st)
+                 : launch_gemm_tile<F4, SWAP, 4, 2, 4>(Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha, st);
 }
 
 template <bool F4>
