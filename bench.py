@@ -513,9 +513,9 @@ def main():
     if (m, n, k) == (8192, 8192, 32768):
         # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE (KiB per dispatch, scaled by a plain 256 MiB
         # copy: x2.0 / x1.0), measured with this script under the profiler: profiles/tnn_gemm_8192x8192x32768_all_engines.md
-        roofline_valu["traffic"] = int((3470626.9 * 2.0 + 288323.6) * 1024)
-        mfma[lib.ENGINE_MFMA_I8]["traffic"] = int((1573450.6 * 2.0 + 262144.0) * 1024)
-        mfma[lib.ENGINE_MFMA_F4]["traffic"] = int((798191.4 * 2.0 + 262144.0) * 1024)
+        roofline_valu["traffic"] = int((2049521.1 * 2.0 + 262183.5) * 1024)
+        mfma[lib.ENGINE_MFMA_I8]["traffic"] = int((1574007.8 * 2.0 + 262144.0) * 1024)
+        mfma[lib.ENGINE_MFMA_F4]["traffic"] = int((790714.8 * 2.0 + 262144.0) * 1024)
     roofline = {lib.ENGINE_VALU: roofline_valu, lib.ENGINE_MFMA_I8: mfma[lib.ENGINE_MFMA_I8],
                 lib.ENGINE_MFMA_F4: mfma[lib.ENGINE_MFMA_F4]}[auto]
 

@@ -109,7 +109,8 @@ template <int MODE, int TM, int TN, int GC, bool IMPL, bool TR = false>
 __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
                                             const uint32_t* __restrict__ B,
                                             float* __restrict__ Y, int M, int KN, int OHW, int G,
-                                            int K_unpack, float alpha, FastDiv dOHW, ConvGeom cg, QuantOut qo) {
+                                            int K_unpack, float alpha, FastDiv dOHW, ConvGeom cg, QuantOut qo,
+                                            int panel) {
     using T = Traits<MODE>;
     constexpr int BM = 64 * TM;
     constexpr int AG = T::kAGroup, BG = T::kBGroup;
@@ -123,8 +124,21 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int64_t row0 = (int64_t)blockIdx.x * BM;
-    const int col0 = (blockIdx.y * 4 + wave) * TN;
+    // Tile of this workgroup.  Large grids are walked in panels of `panel` row tiles: workgroups are dealt to the
+    // eight XCDs round-robin by their linear number, so within a panel an XCD keeps meeting the same panel / 8 row
+    // tiles of A while the column tiles of B stream past -- its private L2 then fetches each A tile once per
+    // round of resident workgroups instead of once per column tile.
+    uint32_t bx = blockIdx.x, by = blockIdx.y;
+    if (panel > 0) {
+        const uint32_t gx = gridDim.x, gy = gridDim.y;
+        const uint32_t lin = bx + gx * by, per = (uint32_t)panel * gy;
+        const uint32_t p = lin / per, within = lin - p * per;
+        const uint32_t pw = min((uint32_t)panel, gx - p * (uint32_t)panel);   // the last panel may be narrower
+        by = within / pw;
+        bx = p * (uint32_t)panel + (within - by * pw);
+    }
+    const int64_t row0 = (int64_t)bx * BM;
+    const int col0 = (by * 4 + wave) * TN;
     const size_t RDA = (size_t)G * AG, RDB = (size_t)G * BG;
 
     uint32_t cn[TM][TN];  // popcount of "negative product" lanes
@@ -371,8 +385,10 @@ hipError_t launch_cfg(const uint32_t* A, const uint32_t* B, float* Y, int64_t M,
     const int cols = qo.mode != 0 ? (KN + 63) / 64 * 64 : KN;
     const int64_t gy = (cols + 4 * TN - 1) / (4 * TN);
     if (gx > 0x7fffffffLL || gy > 65535) return hipErrorInvalidValue;
+    static const int tune_panel = getenv("FTNN_MM_PANEL") ? atoi(getenv("FTNN_MM_PANEL")) : 32;   // tuning aid
+    const int panel = (gx >= 32 && gy >= 32 && gx * gy < 0x7fffffffLL) ? tune_panel : 0;
     hipLaunchKernelGGL((k_mm<MODE, TM, TN, GC, IMPL, TR>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
-                       A, B, Y, (int)M, KN, OHW, G, K_unpack, alpha, make_fastdiv((uint32_t)OHW), cg, qo);
+                       A, B, Y, (int)M, KN, OHW, G, K_unpack, alpha, make_fastdiv((uint32_t)OHW), cg, qo, panel);
     return hipGetLastError();
 }
 

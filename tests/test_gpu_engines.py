@@ -95,6 +95,25 @@ def test_matrix_core_engines_with_256x256_tiles(hip, oracle, typ, shape):
         assert got.tobytes() == want.tobytes(), "engine %d" % eng
 
 
+@pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
+@pytest.mark.parametrize("shape", [(4200, 1, 1, 1100, 4), (7, 30, 29, 1070, 8)], ids=["row_major", "nchw"])
+def test_vector_alu_gemm_walks_large_grids_in_panels(hip, oracle, typ, shape):
+    """grids of 32 x 32 workgroups and more are renumbered into panels of 32 row tiles (the last one narrower when the
+    count is no multiple of 32): every tile must still be computed exactly once"""
+    n, oh, ow, kn, kw = shape
+    m = n * oh * ow
+    rng = np.random.default_rng(5 + typ + kw)
+    at, wt = act_is_ternary(typ), weight_is_ternary(typ)
+    a = rng.integers(-2 ** 63, 2 ** 63, size=m * kw * (2 if at else 1), dtype=np.int64)
+    b = rng.integers(-2 ** 63, 2 ** 63, size=kn * kw * (2 if wt else 1), dtype=np.int64)
+    ku = 64 * kw - 5
+    want = oracle.mm(typ, a, b, n, oh, ow, kn, kw, 0.5, ku)
+    import torch
+    y = torch.full((n, kn, oh, ow), float("nan"), dtype=torch.float32, device="cuda")
+    hip.mm_engine(hip.ENGINE_VALU, typ, _dev(a), _dev(b), n, oh, ow, kn, kw, 0.5, ku, out=y)
+    assert y.cpu().numpy().tobytes() == want.tobytes()
+
+
 def test_lanes_flagged_zero_and_negative_count_as_zero(hip, oracle):
     """a lane with both its sign and its zero bit set is zero in the reference's formula
     (za|zb masks it); the expanded operands must agree"""
