@@ -136,6 +136,64 @@ __device__ __forceinline__ uint2 exchange_halves(uint32_t d0, uint32_t d1) {
     return out;
 }
 
+// PReLU in the reference's two forms: "f <= 0 -> f *= alpha" (TNN, src/tnns/mm_p2_final_tnn_avx2.c:204-208; a zero
+// becomes 0 * alpha) and "r >= 0 ? r : alpha * r" (the others, src/tnns/mm_p2_final_tbn_avx2.c:73)
+template <bool FORM0>
+__device__ __forceinline__ float prelu_ref(float r, float alpha) {
+    const bool scale = FORM0 ? (r <= 0.0f) : (r < 0.0f);
+    return scale ? r * alpha : r;
+}
+
+// One 32-kernel block of a pixel under the hand-over.  r[e] = this lane's 16 results before PReLU, kernel
+// kbase + 8 (e / 4) + 4 h + e % 4 (h = lane half); t = the next layer's threshold for the pixel's image; dq from
+// direct_quant.  Returns the 8 bytes this lane stores at byte 8 h of the block's 16.  Every lane of the wavefront
+// must call it (exchange_halves crosses lanes).
+template <bool FORM0, int QMODE>
+__device__ __forceinline__ uint2 hand_over_block(const float (&r)[16], float alpha, float t, const DirectQuant& dq,
+                                                 int kbase, int h, int KN) {
+    const bool whole = kbase + 32 <= KN;   // wave-uniform: the block holds real kernels only
+    uint32_t d0, d1;
+    if (dq.ok) {
+        // no compares, two nibbles per conversion (see tern_value_direct)
+        const float t_big = t * 0x1p60f;
+        float z[16];
+        if (whole) {
+#pragma unroll
+            for (int e = 0; e < 16; e++) z[e] = direct_value<QMODE>(r[e], alpha, t_big, dq.t_pos, true);
+        } else {   // kernels past KN hold the padding lane
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+                z[e] = direct_value<QMODE>(r[e], alpha, t_big, dq.t_pos, kbase + 8 * (e >> 2) + 4 * h + (e & 3) < KN);
+        }
+        d0 = pack_fp4x8(z[0], z[1], z[2], z[3], z[4], z[5], z[6], z[7]);
+        d1 = pack_fp4x8(z[8], z[9], z[10], z[11], z[12], z[13], z[14], z[15]);
+    } else {
+        constexpr bool tern = QMODE == 1;
+        uint32_t half[4];
+        if (whole) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                half[g] = 0u;
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    half[g] |= quant_nibble(prelu_ref<FORM0>(r[4 * g + i], alpha), t, tern, true) << (4 * i);
+            }
+        } else {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                half[g] = 0u;
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    half[g] |= quant_nibble(prelu_ref<FORM0>(r[4 * g + i], alpha), t, tern, kbase + 8 * g + 4 * h + i < KN)
+                               << (4 * i);
+            }
+        }
+        d0 = half[0] | (half[1] << 16);
+        d1 = half[2] | (half[3] << 16);
+    }
+    return exchange_halves(d0, d1);
+}
+
 // record a failure text for ftnn_last_error(); returns `code`
 int fail(int code, const char* fmt, ...);
 

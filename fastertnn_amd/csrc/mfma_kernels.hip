@@ -504,78 +504,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
             const uint32_t pix = qc - img * (uint32_t)OHW;
             // r = acc - bias: both are integers below 2^24 in fp32, and so is their difference (only BNN has a bias)
             const float fbias = (float)bias;
-            const bool direct = QMODE != 0 && direct_q[b].ok;   // wave-uniform
-            float vals[16];
-            if (!direct) {
+            float r[16];
 #pragma unroll
-                for (int e = 0; e < 16; e++) {
-                    const float fr = FORM0 ? mine[e] : mine[e] - fbias;
-                    // form 0: scale when f <= 0 (a zero becomes 0 * alpha); form 1: scale when r < 0
-                    const bool scale = FORM0 ? (fr <= 0.0f) : (fr < 0.0f);
-                    vals[e] = scale ? fr * alpha : fr;
-                }
-            }
+            for (int e = 0; e < 16; e++) r[e] = FORM0 ? mine[e] : mine[e] - fbias;
             if constexpr (QMODE == 0) {
                 float* yq = Y + ((size_t)img * KN + kn0 + 32 * a + 4 * h) * OHW + pix;
                 if (q < M) {
                     if (kn0 + 32 * a + 32 <= KN) {   // whole block inside: no per-kernel checks
 #pragma unroll
-                        for (int e = 0; e < 16; e++) yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = vals[e];
+                        for (int e = 0; e < 16; e++)
+                            yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = prelu_ref<FORM0>(r[e], alpha);
                     } else {
 #pragma unroll
                         for (int e = 0; e < 16; e++) {
                             const int p = kn0 + 32 * a + 8 * (e >> 2) + 4 * h + (e & 3);
-                            if (p < KN) yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = vals[e];
+                            if (p < KN) yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = prelu_ref<FORM0>(r[e], alpha);
                         }
                     }
                 }
             } else {
-                // Hand-over to an fp4 layer.  Registers 4g .. 4g+3 of this lane are kernels
-                // 8g + 4h + {0..3} of the block: half of nibble dword g of the pixel; the other
-                // half sits in lane ^ 32.  Lane h ends up with dwords 2h and 2h + 1 of the
-                // block's 16 bytes, i.e. bytes 16a + 8h .. + 8 of the pixel's 64-channel word.
-                const float t = qthr[b];
-                constexpr bool tern = QMODE == 1;
-                uint32_t half[4];
-                if (direct) {
-                    // ordinary slope and threshold: no compares, two nibbles per conversion (see tern_value_direct)
-                    const float t_big = t * 0x1p60f;
-                    const bool t_pos = direct_q[b].t_pos;
-                    float z[16];
-                    if (kn0 + 32 * a + 32 <= KN) {   // uniform: the whole block holds real kernels
-#pragma unroll
-                        for (int e = 0; e < 16; e++)
-                            z[e] = direct_value<QMODE>(FORM0 ? mine[e] : mine[e] - fbias, alpha, t_big, t_pos, true);
-                    } else {   // kernels past KN hold the padding lane
-#pragma unroll
-                        for (int e = 0; e < 16; e++)
-                            z[e] = direct_value<QMODE>(FORM0 ? mine[e] : mine[e] - fbias, alpha, t_big, t_pos,
-                                                       kn0 + 32 * a + 8 * (e >> 2) + 4 * h + (e & 3) < KN);
-                    }
-                    const uint32_t d0 = pack_fp4x8(z[0], z[1], z[2], z[3], z[4], z[5], z[6], z[7]);
-                    const uint32_t d1 = pack_fp4x8(z[8], z[9], z[10], z[11], z[12], z[13], z[14], z[15]);
-                    half[0] = d0 & 0xffffu;   // (split and re-joined below at no cost: the compiler folds it)
-                    half[1] = d0 >> 16;
-                    half[2] = d1 & 0xffffu;
-                    half[3] = d1 >> 16;
-                } else if (kn0 + 32 * a + 32 <= KN) {   // uniform: the whole block holds real kernels
-#pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        half[g] = 0u;
-#pragma unroll
-                        for (int i = 0; i < 4; i++) half[g] |= quant_nibble(vals[4 * g + i], t, tern, true) << (4 * i);
-                    }
-                } else {
-#pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        half[g] = 0u;
-#pragma unroll
-                        for (int i = 0; i < 4; i++)
-                            half[g] |= quant_nibble(vals[4 * g + i], t, tern, kn0 + 32 * a + 8 * g + 4 * h + i < KN)
-                                       << (4 * i);
-                    }
-                }
-                const uint2 out = exchange_halves(half[0] | (half[1] << 16), half[2] | (half[3] << 16));
+                // Hand-over to an fp4 layer.  Registers 4g .. 4g+3 of this lane are kernels 8g + 4h + {0..3} of the
+                // block: half of nibble dword g of the pixel, the other half sits in lane ^ 32.  Lane half h ends up
+                // with bytes 16a + 8h .. + 8 of the pixel's 64-channel word.
+                const uint2 out = hand_over_block<FORM0, QMODE>(r, alpha, qthr[b], direct_q[b], kn0 + 32 * a, h, KN);
                 const size_t word = ((size_t)img * gridDim.y + blockIdx.y) * OHW + pix;
                 if (q < M) *reinterpret_cast<uint2*>(static_cast<unsigned char*>(qo.p4) + word * 32 + 16 * a + 8 * h) = out;
             }
@@ -689,61 +640,25 @@ __global__ __launch_bounds__(256) void k_conv_f4_small(const uint4* __restrict__
 
     // accumulator e: kernel = kn0 + 8*(e/4) + 4*h + e%4, pixel = px0 + lr
     const float fbias = (float)bias;
-    const bool whole = kn0 + 32 <= KN;   // uniform
-    const DirectQuant dq = direct_quant<QMODE>(alpha, qthr);
-    const bool direct = QMODE != 0 && dq.ok;
-    float vals[16];
-    if (!direct) {
+    float r[16];
 #pragma unroll
-        for (int e = 0; e < 16; e++) {
-            const float fr = FORM0 ? acc[e] : acc[e] - fbias;
-            const bool scale = FORM0 ? (fr <= 0.0f) : (fr < 0.0f);
-            vals[e] = scale ? fr * alpha : fr;
-        }
-    }
+    for (int e = 0; e < 16; e++) r[e] = FORM0 ? acc[e] : acc[e] - fbias;   // only BNN has a bias
     if constexpr (QMODE == 0) {
         float* yq = Y + ((size_t)img * KN + kn0 + 4 * h) * OHW + pix;
         if (q < M) {
-            if (whole) {
+            if (kn0 + 32 <= KN) {   // uniform: whole block inside
 #pragma unroll
-                for (int e = 0; e < 16; e++) yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = vals[e];
+                for (int e = 0; e < 16; e++) yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = prelu_ref<FORM0>(r[e], alpha);
             } else {
 #pragma unroll
                 for (int e = 0; e < 16; e++) {
                     const int p = kn0 + 8 * (e >> 2) + 4 * h + (e & 3);
-                    if (p < KN) yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = vals[e];
+                    if (p < KN) yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = prelu_ref<FORM0>(r[e], alpha);
                 }
             }
         }
     } else {
-        constexpr bool tern = QMODE == 1;
-        uint32_t d0, d1;
-        if (direct) {
-            const float t_big = qthr * 0x1p60f;
-            float z[16];
-#pragma unroll
-            for (int e = 0; e < 16; e++)
-                z[e] = direct_value<QMODE>(FORM0 ? acc[e] : acc[e] - fbias, alpha, t_big, dq.t_pos, true);
-            if (!whole) {   // kernels past KN: the padding lane
-#pragma unroll
-                for (int e = 0; e < 16; e++)
-                    z[e] = kn0 + 8 * (e >> 2) + 4 * h + (e & 3) < KN ? z[e] : (QMODE == 1 ? 0.0f : 1.0f);
-            }
-            d0 = pack_fp4x8(z[0], z[1], z[2], z[3], z[4], z[5], z[6], z[7]);
-            d1 = pack_fp4x8(z[8], z[9], z[10], z[11], z[12], z[13], z[14], z[15]);
-        } else {
-            uint32_t half[4];
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                half[g] = 0u;
-#pragma unroll
-                for (int i = 0; i < 4; i++)
-                    half[g] |= quant_nibble(vals[4 * g + i], qthr, tern, whole || kn0 + 8 * g + 4 * h + i < KN) << (4 * i);
-            }
-            d0 = half[0] | (half[1] << 16);
-            d1 = half[2] | (half[3] << 16);
-        }
-        const uint2 out = exchange_halves(d0, d1);
+        const uint2 out = hand_over_block<FORM0, QMODE>(r, alpha, qthr, direct_quant<QMODE>(alpha, qthr), kn0, h, KN);
         // this tile is half a 64-channel word: bytes 16 * (tile parity) of the pixel's 32
         const size_t word = ((size_t)img * (gridDim.y >> 1) + (blockIdx.y >> 1)) * OHW + pix;
         if (q < M)

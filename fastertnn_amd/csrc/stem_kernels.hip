@@ -204,81 +204,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
     const float fbias = (float)bias;
     float qthr = 0.0f;
     if constexpr (QMODE != 0) qthr = qo.thr[n];
-    // hand-over with an ordinary slope and threshold: the nibbles come straight from the accumulators
-    const DirectQuant dq = direct_quant<QMODE>(alpha, qthr);
-    const bool direct = QMODE != 0 && dq.ok;
-    const float qthr_big = qthr * 0x1p60f;
+    const DirectQuant dq = direct_quant<QMODE>(alpha, qthr);   // whether the hand-over may take its compare-free form
 #pragma unroll
     for (int a = 0; a < 2; a++)
 #pragma unroll
         for (int b = 0; b < 2; b++) {
             const bool live = oh[b] < g.OH && ow[b] < g.OW;
             const int pix = live ? oh[b] * g.OW + ow[b] : 0;
-            const bool whole = kn0 + 32 * a + 32 <= KN;   // uniform: the block holds real kernels only
-            float vals[16];
-            if (!direct) {
+            float r[16];
 #pragma unroll
-                for (int e = 0; e < 16; e++) {
-                    const float fr = FORM0 ? acc[a][b][e] : acc[a][b][e] - fbias;   // only BNN has a bias
-                    const bool scale = FORM0 ? (fr <= 0.0f) : (fr < 0.0f);
-                    vals[e] = scale ? fr * alpha : fr;
-                }
-            }
+            for (int e = 0; e < 16; e++) r[e] = FORM0 ? acc[a][b][e] : acc[a][b][e] - fbias;   // only BNN has a bias
             if constexpr (QMODE == 0) {
                 float* yq = Y + ((size_t)n * KN + kn0 + 32 * a + 4 * h) * OHW + pix;
                 if (live) {
-                    if (whole) {
+                    if (kn0 + 32 * a + 32 <= KN) {   // uniform: whole block inside
 #pragma unroll
-                        for (int e = 0; e < 16; e++) yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = vals[e];
+                        for (int e = 0; e < 16; e++)
+                            yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = prelu_ref<FORM0>(r[e], alpha);
                     } else {
 #pragma unroll
                         for (int e = 0; e < 16; e++) {
                             const int p = kn0 + 32 * a + 8 * (e >> 2) + 4 * h + (e & 3);
-                            if (p < KN) yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = vals[e];
+                            if (p < KN) yq[(size_t)(8 * (e >> 2) + (e & 3)) * OHW] = prelu_ref<FORM0>(r[e], alpha);
                         }
                     }
                 }
             } else {
-                // the same exchange as in k_conv_f4: lane h ends up with bytes 16 a + 8 h .. + 8 of the pixel's word
-                constexpr bool tern = QMODE == 1;
-                uint32_t half[4];
-                if (direct) {
-                    float z[16];
-                    if (whole) {
-#pragma unroll
-                        for (int e = 0; e < 16; e++)
-                            z[e] = direct_value<QMODE>(FORM0 ? acc[a][b][e] : acc[a][b][e] - fbias, alpha, qthr_big,
-                                                       dq.t_pos, true);
-                    } else {   // kernels past KN: the padding lane
-#pragma unroll
-                        for (int e = 0; e < 16; e++)
-                            z[e] = direct_value<QMODE>(FORM0 ? acc[a][b][e] : acc[a][b][e] - fbias, alpha, qthr_big,
-                                                       dq.t_pos, kn0 + 32 * a + 8 * (e >> 2) + 4 * h + (e & 3) < KN);
-                    }
-                    const uint32_t d0 = pack_fp4x8(z[0], z[1], z[2], z[3], z[4], z[5], z[6], z[7]);
-                    const uint32_t d1 = pack_fp4x8(z[8], z[9], z[10], z[11], z[12], z[13], z[14], z[15]);
-                    half[0] = d0 & 0xffffu;   // (split and re-joined below at no cost: the compiler folds it)
-                    half[1] = d0 >> 16;
-                    half[2] = d1 & 0xffffu;
-                    half[3] = d1 >> 16;
-                } else if (whole) {
-#pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        half[q] = 0u;
-#pragma unroll
-                        for (int i = 0; i < 4; i++) half[q] |= quant_nibble(vals[4 * q + i], qthr, tern, true) << (4 * i);
-                    }
-                } else {
-#pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        half[q] = 0u;
-#pragma unroll
-                        for (int i = 0; i < 4; i++)
-                            half[q] |= quant_nibble(vals[4 * q + i], qthr, tern, kn0 + 32 * a + 8 * q + 4 * h + i < KN)
-                                       << (4 * i);
-                    }
-                }
-                const uint2 out = exchange_halves(half[0] | (half[1] << 16), half[2] | (half[3] << 16));
+                // as in k_conv_f4: lane half h ends up with bytes 16 a + 8 h .. + 8 of the pixel's 64-channel word
+                const uint2 out = hand_over_block<FORM0, QMODE>(r, alpha, qthr, dq, kn0 + 32 * a, h, KN);
                 const size_t word = ((size_t)n * gridDim.y + blockIdx.y) * OHW + pix;
                 if (live)
                     *reinterpret_cast<uint2*>(static_cast<unsigned char*>(qo.p4) + word * 32 + 16 * a + 8 * h) = out;
