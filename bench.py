@@ -368,6 +368,50 @@ def reference_gemm_sweep(torch, lib, reps=10):
     return out
 
 
+def reference_single_layers(torch, lib, batch=8, reps=10):
+    """the 17 layers of the reference's `layer` mode (include/timing/shapes_layers.h, kept as data in
+    tests/golden/reference_shape_tables.json), TNN, batch 8 (src/timing_layers.c:46): device-resident call with
+    prepared weights against the reference's tnns_conv on one host core"""
+    import numpy as np
+    from fastertnn_amd import TNN
+    from oracle import ftnn_oracle as O
+    tables = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "golden",
+                                         "reference_shape_tables.json")))
+    out = {}
+    g = torch.Generator(device="cuda")
+    g.manual_seed(9)
+    for shape in tables["layers"]:
+        c, ih, iw, kn, kw, kh, p, s = shape
+        x = torch.randn((batch, c, ih, iw), generator=g, device="cuda")
+        thr = torch.full((batch,), 0.5, device="cuda")
+        w = torch.randint(-1, 2, (kn, c, kh, kw), generator=g, device="cuda", dtype=torch.int8).float()
+        qw = lib.pack_weights(w, torch.full((kn,), 0.5, device="cuda"), True)
+        del w
+        prepared = lib.prepare_conv_weights(TNN, qw, c, kn, kh, kw)
+        oh, ow = lib.out_dim(ih, p, kh, s), lib.out_dim(iw, p, kw, s)
+        scratch = torch.empty(lib.conv_scratch_bytes(TNN, batch, c, ih, iw, kn, kh, kw, p, s), dtype=torch.uint8,
+                              device="cuda")
+        y = torch.empty((batch, kn, oh, ow), device="cuda")
+
+        def step():
+            lib.conv_prepared(TNN, x, thr, prepared, kn, kh, kw, p, s, 0.5, scratch=scratch, out=y)
+        for _ in range(3):
+            step()
+        t = sorted(event_times(torch, step, reps))[reps // 2]
+        row = {"engine": lib.ENGINE_NAMES[lib.select_conv_engine(TNN, batch, c, ih, iw, kn, kh, kw, p, s)],
+               "device_ms": round(t, 4), "gmac": round(batch * oh * ow * kn * c * kh * kw / 1e9, 2)}
+        if O.Reference.available():
+            ref = O.Reference()
+            xh, qwh = x.cpu().numpy(), O.aligned_copy(qw.cpu().numpy())
+            t0 = time.perf_counter()
+            want = ref.conv(TNN, xh, np.full(batch, 0.5, np.float32), qwh, kn, kh, kw, p, s, 0.5)
+            row["cpu_ms"] = round((time.perf_counter() - t0) * 1e3, 2)
+            row["bit_exact_vs_reference"] = bool(y.cpu().numpy().tobytes() == np.ascontiguousarray(want).tobytes())
+        out["c%d_%dx%d_k%d_s%d" % (c, ih, iw, kh, s)] = row
+        del x, qw, prepared, scratch, y
+    return out
+
+
 def reference_networks(torch, lib, batch=8, reps=5):
     """the networks of the reference's e2e mode that chain shape to shape (include/timing/shapes_e2e.h, kept as
     data in tests/golden/reference_shape_tables.json), at the reference's batch of 8 (src/timing_layers.c:46):
@@ -544,6 +588,7 @@ def main():
             "tnn_resnet18_like_b32_e2e": e2e_latency(torch, lib, 32),
             "valu_popcount_probe": valu_probe(),
             "reference_gemm_sweep": reference_gemm_sweep(torch, lib),
+            "reference_single_layers_b8": reference_single_layers(torch, lib),
             "reference_e2e_networks_b8": reference_networks(torch, lib),
             "tnn_resnet18_like_other_batches": {"b%d" % b: e2e_latency(torch, lib, b, cpu=False) for b in (1, 8, 128)},
             "other_types_resnet18_like_b32": {n: e2e_latency(torch, lib, 32, cpu=False, typ=t)

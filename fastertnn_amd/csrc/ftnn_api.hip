@@ -178,9 +178,35 @@ int64_t conv_f4_dense_bytes(int N, int C, int H, int W, int KH, int KW, int OH, 
     return dense_f4_pq_bytes(N, H, W) + ((int64_t)N * OH * OW * Kd * 32 + 255) / 256 * 256;
 }
 
-// operand region of the fp4 layer for this shape, whichever of the two forms it takes
-int64_t conv_f4_operand_bytes(int N, int C, int H, int W, int KH, int KW, int OH, int OW) {
-    return dense_f4_applies(C, KH, KW) ? conv_f4_dense_bytes(N, C, H, W, KH, KW, OH, OW) : conv_f4_p4_bytes(N, C, H, W);
+// Large layers with an fp32 result run as quantise + im2row + expansion + the GEMM kernel with LDS-staged 128 / 256
+// tiles: from about 12 GMAC, with tiles for every compute unit, the layer kernel's wavefronts, each fetching its own
+// fragments through the L1, fall behind it (the reference's 1024-channel 56 x 56 layer at batch 8, 59 GMAC: 139 us
+// against 80 us; 15 GMAC layers with 100-200 tiles are a tie).
+bool conv_f4_gemm_route(int64_t M, int KN, int K) {
+    static const bool off = getenv("FTNN_CONV_NO_GEMM_ROUTE") != nullptr;   // tuning aid
+    // enough 128 x 128 tiles for every compute unit, and enough work to pay for the three extra passes
+    const int64_t tiles = ((M + 127) / 128) * ((KN + 127) / 128);
+    return !off && tiles >= 256 && M <= 0x7fffffffLL && (double)M * KN * 64.0 * K >= 1.2e10;
+}
+
+// its buffers: channel-packed planes, Packing-2 rows, the rows as matrix-core fragments (each 256-byte aligned)
+static int64_t gemm_route_plane_bytes(int N, int C, int H, int W) {
+    return (ftnn_pack_scratch_bytes(N, C, H, W, 1) + 255) / 256 * 256;
+}
+static int64_t gemm_route_row_bytes(int64_t M, int Kw) { return (M * Kw * 16 + 255) / 256 * 256; }
+
+// operand region of the fp4 layer for this shape, whichever form it takes
+int64_t conv_f4_operand_bytes(int N, int C, int H, int W, int KH, int KW, int OH, int OW, int KN) {
+    if (dense_f4_applies(C, KH, KW)) return conv_f4_dense_bytes(N, C, H, W, KH, KW, OH, OW);
+    int64_t bytes = conv_f4_p4_bytes(N, C, H, W);
+    const int64_t M = (int64_t)N * OH * OW;
+    if (conv_f4_gemm_route(M, KN, cpack_of(C) * KH * KW)) {
+        const int Kw = conv_f4_weight_words(C, KH, KW);
+        const int64_t route = gemm_route_plane_bytes(N, C, H, W) + gemm_route_row_bytes(M, Kw) +
+                              (mfma_fragment_bytes(true, M, Kw) + 255) / 256 * 256;
+        if (route > bytes) bytes = route;
+    }
+    return bytes;
 }
 
 // words per expanded weight row on the fp4 layer path
@@ -220,6 +246,20 @@ int conv_f4_expanded(int type, const float* d_x, const float* d_thr, const void*
                              make_fastdiv((uint32_t)OW), make_fastdiv((uint32_t)Kd), make_fastdiv(1u)};
         e = launch_conv_f4(type, d_a4, d_wf, cg, N, KN, C * KH * KW, prelu_alpha, d_y, st, qo);
         return e == hipSuccess ? FTNN_OK : hip_fail(e, "fp4 conv launch");
+    }
+    const int64_t M = (int64_t)N * OH * OW;
+    if (d_x && qo.mode == 0 && conv_f4_gemm_route(M, KN, cpack_of(C) * KH * KW)) {
+        const int Kw = conv_f4_weight_words(C, KH, KW);
+        char* base = static_cast<char*>(d_p4);
+        int64_t* d_rows = reinterpret_cast<int64_t*>(base + gemm_route_plane_bytes(N, C, H, W));
+        void* d_af = reinterpret_cast<char*>(d_rows) + gemm_route_row_bytes(M, Kw);
+        e = launch_quantize_im2row(act_ternary, d_x, d_thr, N, C, H, W, H_pad, W_pad, KH, KW, H_stride, W_stride, d_rows,
+                                   base, st);
+        if (e != hipSuccess) return hip_fail(e, "quantise + im2row launch");
+        e = launch_mfma_expand(true, act_ternary, d_rows, (int)M, Kw, d_af, st);
+        if (e != hipSuccess) return hip_fail(e, "row expansion launch");
+        e = launch_mfma_gemm(true, type, d_af, d_wf, M, OH * OW, KN, Kw, C * KH * KW, prelu_alpha, d_y, st);
+        return e == hipSuccess ? FTNN_OK : hip_fail(e, "matrix-core GEMM launch");
     }
     if (d_x) e = launch_quantize_f4(act_ternary, d_x, d_thr, N, C, H, W, d_p4, st);   // else d_p4 is ready
     if (e != hipSuccess) return hip_fail(e, "fp4 quantize launch");
@@ -322,7 +362,7 @@ int64_t ftnn_conv_scratch_bytes(int type, int N, int C, int H, int W, int KN, in
     }
     // enough for either engine, so that one buffer serves ftnn_conv and ftnn_conv_engine
     // fp4: operand region, fragments of the weights and, on the dense path, the re-packed weight rows
-    int64_t f4 = conv_f4_operand_bytes(N, C, H, W, KH, KW, OH, OW) +
+    int64_t f4 = conv_f4_operand_bytes(N, C, H, W, KH, KW, OH, OW, KN) +
                  (mfma_fragment_bytes(true, KN, conv_f4_weight_words(C, KH, KW)) + 255) / 256 * 256;
     if (dense_f4_applies(C, KH, KW)) f4 += (int64_t)KN * conv_f4_weight_words(C, KH, KW) * (wt ? 16 : 8);
     return bytes > f4 ? bytes : f4;
@@ -483,7 +523,7 @@ int ftnn_conv_engine(int engine, int type, const float* d_x, const float* d_thr,
         if (64LL * Kw >= (1LL << 24))
             return fail(FTNN_EINVAL, "K too long for exact fp32 accumulation; use the vector-ALU engine");
         if (!fits_f4) return fail(FTNN_EINVAL, "more than 2^31-1 input pixel words: use the vector-ALU engine");
-        char* d_wf = static_cast<char*>(d_scratch) + conv_f4_operand_bytes(N, C, H, W, KH, KW, OH, OW);
+        char* d_wf = static_cast<char*>(d_scratch) + conv_f4_operand_bytes(N, C, H, W, KH, KW, OH, OW, KN);
         const int64_t* rows = d_qw;
         hipError_t e;
         if (dense_f4_applies(C, KH, KW)) {   // the weights take the same re-packing first

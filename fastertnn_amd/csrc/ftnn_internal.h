@@ -274,7 +274,7 @@ int conv_valu(int type, const float* d_x, const float* d_thr, const int64_t* d_q
               void* d_scratch, float* d_y, hipStream_t st, const QuantOut& qo, bool weights_prepared);
 // bytes of the fp4 layer's operand region (d_p4 above) for this shape, rounded up to 256: P4, or for a
 // few-channel layer the nibble pixels and dense rows
-int64_t conv_f4_operand_bytes(int N, int C, int H, int W, int KH, int KW, int OH, int OW);
+int64_t conv_f4_operand_bytes(int N, int C, int H, int W, int KH, int KW, int OH, int OW, int KN);
 // words per row of the weights as the fp4 layer reads them (the dense re-packing shortens them)
 int conv_f4_weight_words(int C, int KH, int KW);
 

@@ -129,7 +129,7 @@ ftnn_net_t* ftnn_net_create(int batch, int n_layers, const ftnn_layer_t* layers)
                       (int64_t)batch * net->OH[i] * net->OW[i] * conv_f4_weight_words(L.C, L.KH, L.KW) > 0x7fffffffLL))
             f4[i] = 0;   // beyond the 32-bit pixel indices of the fp4 layer kernel: the vector-ALU layer takes it
         if (f4[i]) {
-            max_p4 = std::max(max_p4, conv_f4_operand_bytes(batch, L.C, L.H, L.W, L.KH, L.KW, net->OH[i], net->OW[i]));
+            max_p4 = std::max(max_p4, conv_f4_operand_bytes(batch, L.C, L.H, L.W, L.KH, L.KW, net->OH[i], net->OW[i], L.KN));
             if (i > 0 && dense_f4_applies(L.C, L.KH, L.KW))   // its input arrives as fp32
                 max_act = std::max(max_act, (int64_t)batch * L.C * L.H * L.W);
         } else {

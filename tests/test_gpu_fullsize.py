@@ -144,3 +144,31 @@ def test_nchw_results_beyond_2_32_elements(hip, oracle):
         hip.mm_engine(eng, TNN, rows, qw, n, hw, hw, kn, 9, 0.5, out=y)
         assert torch.equal(y, ref), "gemm engine %d" % eng
         del y
+
+
+@pytest.mark.parametrize("typ", [TNN, TBN, BTN, BNN], ids=lambda t: TYPE_NAMES[t])
+def test_large_layer_takes_the_gemm_route(hip, oracle, typ):
+    """a 29.6 GMAC layer (batch 16, 512 -> 512 channels at 28 x 28, 392 tiles of 128 x 128): the fp4 engine runs it as quantise + im2row +
+    expansion + the tiled GEMM kernel.  Same bits as the vector-ALU engine on every element, and as the oracle on
+    one image"""
+    import torch
+    from fastertnn_amd import synth
+    n, c, hw, kn = 16, 512, 28, 512
+    assert ((n * hw * hw + 127) // 128) * ((kn + 127) // 128) >= 256
+    at, wt = act_is_ternary(typ), weight_is_ternary(typ)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(31 + typ)
+    x = torch.randn((n, c, hw, hw), generator=g, device="cuda")
+    thr = torch.full((n,), 0.5 if at else 0.0, device="cuda")
+    w = synth.ternary(40 + typ, (kn, c, 3, 3)) if wt else synth.binary(40 + typ, (kn, c, 3, 3))
+    qw_h = oracle.pack_weights(w, np.full(kn, 0.5 if wt else 0.0, np.float32), wt)
+    qw = torch.from_numpy(qw_h).cuda()
+    got = hip.conv(typ, x, thr, qw, kn, 3, 3, 1, 1, 0.5, engine=hip.ENGINE_MFMA_F4)
+    ref = hip.conv(typ, x, thr, qw, kn, 3, 3, 1, 1, 0.5, engine=hip.ENGINE_VALU)
+    assert torch.equal(got, ref)
+    want = oracle.conv(typ, x[5:6].cpu().numpy(), np.full(1, 0.5 if at else 0.0, np.float32), qw_h, kn, 3, 3, 1, 1, 0.5)
+    assert got[5:6].cpu().numpy().tobytes() == np.ascontiguousarray(want).tobytes()
+    # prepared weights take the same route
+    prepared = hip.prepare_conv_weights(typ, qw, c, kn, 3, 3)
+    got2 = hip.conv_prepared(typ, x, thr, prepared, kn, 3, 3, 1, 1, 0.5)
+    assert torch.equal(got2, ref)
