@@ -160,3 +160,15 @@ def test_popcount_probe_is_built_beside_the_library():
     from fastertnn_amd import build
     assert os.path.exists(build.LIB)
     assert os.access(build.PROBE, os.X_OK)
+
+
+def test_size_limits_need_no_device():
+    """shapes beyond the documented limits are refused (a scratch size of 0 is how the size query says so)"""
+    import fastertnn_amd.lib as lib
+    assert lib.conv_scratch_bytes(0, 1, 1, 8192, 8191, 1, 1, 1, 0, 1) > 0         # just below 2^26 pixels per plane
+    assert lib.conv_scratch_bytes(0, 1, 1, 8192, 8192, 1, 1, 1, 0, 1) == 0        # 2^26: refused
+    assert lib.conv_scratch_bytes(0, 65536, 1, 4, 4, 1, 1, 1, 0, 1) == 0          # batch above 65535
+    # a very large layer sizes its scratch for the im2row + GEMM form: planes + rows + fragments
+    big = lib.conv_scratch_bytes(0, 8, 1024, 56, 56, 1024, 3, 3, 1, 2)
+    small = lib.conv_scratch_bytes(0, 8, 1024, 56, 56, 128, 3, 3, 1, 2)
+    assert big > small > 0
