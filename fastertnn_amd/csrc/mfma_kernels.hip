@@ -757,8 +757,7 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
     // alone do that (a tile = 64 kernels x 64 pixels)
     const int64_t tiles = ((M + 63) / 64) * ((KN + 63) / 64);
     int split = tiles >= 600 ? 1 : (tiles >= 450 ? 2 : 4);   // measured on MI355X (1024 SIMDs)
-    static const int min_words = getenv("FTNN_CONV_SPLIT_MIN_WORDS") ? atoi(getenv("FTNN_CONV_SPLIT_MIN_WORDS")) : 1;
-    while (split > 1 && cg.K < min_words * split) split /= 2;   // no wavefront without K words of its own
+    while (split > 1 && cg.K < split) split /= 2;   // no wavefront without K words of its own
     static const char* tune = getenv("FTNN_CONV_SPLIT");   // tuning aid: force the K split
     if (tune) split = atoi(tune);
     const int wpb = 4, tpb = wpb / split;   // wavefronts and pixel tiles per workgroup (see the kernel)
