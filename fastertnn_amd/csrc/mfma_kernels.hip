@@ -56,25 +56,40 @@ struct Tile {
 template <bool F4, bool TERN>
 __global__ __launch_bounds__(256) void k_expand(const uint32_t* __restrict__ P, int rows, int G,
                                                 uint4* __restrict__ out) {
-    // a workgroup expands kGPB adjacent groups of its 32 rows: 256 contiguous bytes of each ternary row, so
-    // that both halves of a 128-byte line are consumed by the same workgroup, with all loads issued up front
+    // A workgroup expands kGPB adjacent groups of its 32 rows: 256 contiguous bytes of each ternary row (128 of a
+    // binary one).  They are fetched row-wise, 16 bytes per thread with neighbouring threads on neighbouring bytes,
+    // and turned through LDS into the (row, dword) order the expansion works in: fetched in that order directly,
+    // every load instruction would touch 32 cache lines for 256 bytes.
     constexpr int kGPB = 4;
+    constexpr int DPG = TERN ? 16 : 8;        // dwords per group and row
+    constexpr int RD = kGPB * DPG;            // dwords per row in the block: 64 / 32
+    constexpr int RS = RD + 1;                // LDS row stride: odd, the 32 rows of a read hit 32 banks
+    __shared__ uint32_t stage[32 * RS];
     const int rb = blockIdx.x, g0 = blockIdx.y * kGPB, t = threadIdx.x;
+    {
+        constexpr int PPR = RD / 4;           // 16-byte pieces per row: 16 / 8
+        const int gmax = min(kGPB, G - g0) * (DPG / 4);   // pieces of a row that exist
+#pragma unroll
+        for (int k = 0; k < (32 * PPR) / 256; k++) {
+            const int idx = t + 256 * k, rr = idx / PPR, pc = idx - rr * PPR;
+            const int srow = min(rb * 32 + rr, rows - 1);
+            uint4 v = make_uint4(0u, 0u, 0u, 0u);
+            if (pc < gmax) v = *reinterpret_cast<const uint4*>(P + ((size_t)srow * G + g0) * DPG + pc * 4);
+            uint32_t* d = stage + rr * RS + pc * 4;
+            d[0] = v.x;
+            d[1] = v.y;
+            d[2] = v.z;
+            d[3] = v.w;
+        }
+    }
+    __syncthreads();
     const int r = t & 31, dq = t >> 5;
-    const int row = min(rb * 32 + r, rows - 1);
     const bool live = rb * 32 + r < rows;
     uint32_t sv[kGPB], zv[kGPB];
 #pragma unroll
     for (int i = 0; i < kGPB; i++) {
-        const int g = min(g0 + i, G - 1);
-        if (TERN) {
-            const uint32_t* src = P + ((size_t)row * G + g) * 16;
-            sv[i] = src[dq];
-            zv[i] = src[8 + dq];
-        } else {
-            sv[i] = P[((size_t)row * G + g) * 8 + dq];
-            zv[i] = 0u;
-        }
+        sv[i] = stage[r * RS + i * DPG + dq];
+        zv[i] = TERN ? stage[r * RS + i * DPG + 8 + dq] : 0u;
     }
 #pragma unroll
     for (int i = 0; i < kGPB; i++) {
