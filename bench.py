@@ -69,6 +69,19 @@ def event_times(torch, fn, reps):
     return [a.elapsed_time(b) for a, b in ev]
 
 
+def host_cpu():
+    """the host the CPU baseline ran on: model name and the cores present (the baseline itself uses one)"""
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return {"model": model, "cores_present": os.cpu_count()}
+
+
 def cpu_gemm_baseline(a_host, b_host, rows, n, kw, alpha):
     """reference mm_tnn on one core (its protocol pins the process to core 0, Makefile:21);
     falls back to the plain-C port when the compiled reference is absent"""
@@ -574,7 +587,8 @@ def main():
         cpu = {"value": round(float(rows) * n * k / dt / 1e9, 2), "unit": "GMAC/s", "cores": 1, "kind": kind,
                "sample": "first %d of %d rows of A against all %d columns, K=%d (%.1f s on one core)"
                          % (rows, m, n, k, dt),
-               "gpu_rows_bit_exact": bool(y_gpu.tobytes() == np.ascontiguousarray(y_cpu).tobytes())}
+               "gpu_rows_bit_exact": bool(y_gpu.tobytes() == np.ascontiguousarray(y_cpu).tobytes()),
+               "host": host_cpu()}
 
     extra = None
     if not args.no_extra:
