@@ -28,19 +28,26 @@ static int hip_fail(hipError_t e, const char* what) {
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// words per operand row (one plane) that every engine's 32-bit sums and offsets hold
+constexpr int kMaxRowWords = (1 << 24) - 4;
+
 // common conv-shape validation; fills OH/OW
-static int check_conv_shape(int N, int C, int H, int W, int H_pad, int W_pad, int kH, int kW,
+int check_conv_shape(int N, int C, int H, int W, int H_pad, int W_pad, int kH, int kW,
                             int H_stride, int W_stride, int* OH, int* OW) {
     if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || kH <= 0 || kW <= 0 || H_stride <= 0 ||
         W_stride <= 0 || H_pad < 0 || W_pad < 0)
         return fail(FTNN_EINVAL, "non-positive dimension or negative padding");
-    if (H + 2 * H_pad < kH || W + 2 * W_pad < kW)
-        return fail(FTNN_EINVAL, "kernel %dx%d larger than padded input %dx%d", kH, kW,
-                    H + 2 * H_pad, W + 2 * W_pad);
+    const int64_t Hp = (int64_t)H + 2 * (int64_t)H_pad, Wp = (int64_t)W + 2 * (int64_t)W_pad;
+    if (Hp < kH || Wp < kW)
+        return fail(FTNN_EINVAL, "kernel %dx%d larger than padded input %lldx%lld", kH, kW, (long long)Hp,
+                    (long long)Wp);
     if (N > 65535) return fail(FTNN_EINVAL, "batch %d above the supported 65535", N);
     // pixel indices within one image plane are 32-bit in the kernels (27 of them in one store offset)
-    if (((int64_t)H + 2 * H_pad) * ((int64_t)W + 2 * W_pad) > 0x3ffffffLL)
+    if (Hp > 0x3ffffffLL || Wp > 0x3ffffffLL || Hp * Wp > 0x3ffffffLL)
         return fail(FTNN_EINVAL, "padded image plane above the supported 2^26 pixels");
+    // 32-bit accumulators count up to 128 per word of a row
+    if (C > (1 << 30) || ((int64_t)C + 63) / 64 * kH * kW > kMaxRowWords)
+        return fail(FTNN_EINVAL, "more than %d words per im2row row", kMaxRowWords);
     *OH = out_dim(H, H_pad, kH, H_stride);
     *OW = out_dim(W, W_pad, kW, W_stride);
     return FTNN_OK;
@@ -143,8 +150,8 @@ static int64_t* host_quantize_im2row(bool ternary, float* x, float* thr, int N, 
 static float* host_mm(int type, int64_t* a, int64_t* b, int N, int OH, int OW, int KN, int K,
                       int K_unpack, float alpha) {
     std::lock_guard<std::mutex> lock(g_ctx_mutex);
-    if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0) {
-        fail(FTNN_EINVAL, "non-positive GEMM dimension");
+    if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0 || K > kMaxRowWords) {
+        fail(FTNN_EINVAL, "GEMM dimension non-positive or K above %d words", kMaxRowWords);
         die("mm");
     }
     const size_t M = (size_t)N * OH * OW;
@@ -320,7 +327,10 @@ const char* ftnn_version(void) { return "ftnn-hip 0.1 gfx950"; }
 int ftnn_out_dim(int in, int pad, int k, int stride) { return out_dim(in, pad, k, stride); }
 
 int64_t ftnn_row_words(int C, int KH, int KW, int ternary) {
-    const int64_t kw = round4(cpack_of(C) * KH * KW);
+    if (C <= 0 || KH <= 0 || KW <= 0) return 0;
+    const int64_t k = ((int64_t)C + 63) / 64 * KH * KW;
+    if (k > kMaxRowWords) return 0;
+    const int64_t kw = (k + 3) / 4 * 4;
     return ternary ? 2 * kw : kw;
 }
 
@@ -388,6 +398,7 @@ int ftnn_mm(int type, const int64_t* d_a, const int64_t* d_b, int N, int OH, int
     if (type < kTNN || type > kBNN) return fail(FTNN_EINVAL, "unknown network type %d", type);
     if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0)
         return fail(FTNN_EINVAL, "non-positive GEMM dimension");
+    if (K > kMaxRowWords) return fail(FTNN_EINVAL, "K = %d words above the supported %d", K, kMaxRowWords);
     if (!d_a || !d_b || !d_y) return fail(FTNN_EINVAL, "null device pointer");
     if (!aligned16(d_a) || !aligned16(d_b))
         return fail(FTNN_EINVAL, "GEMM operands must be 16-byte aligned");
@@ -413,12 +424,12 @@ static int select_engine(int type, int64_t M, int KN, int Kw) {
 }
 
 int ftnn_select_engine(int type, int N, int OH, int OW, int KN, int K) {
-    if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0) return FTNN_ENGINE_VALU;
+    if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0 || K > kMaxRowWords) return FTNN_ENGINE_VALU;
     return select_engine(type, (int64_t)N * OH * OW, KN, round4(K));
 }
 
 int64_t ftnn_mm_scratch_bytes(int engine, int type, int N, int OH, int OW, int KN, int K) {
-    if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0) return 0;
+    if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0 || K > kMaxRowWords) return 0;
     const int64_t M = (int64_t)N * OH * OW;
     const int Kw = round4(K);
     if (engine == FTNN_ENGINE_AUTO) engine = select_engine(type, M, KN, Kw);
@@ -436,13 +447,13 @@ static int check_mfma_engine(int engine, int Kw) {
 }
 
 int64_t ftnn_expand_bytes(int engine, int rows, int K) {
-    if (rows <= 0 || K <= 0 || (engine != FTNN_ENGINE_MFMA_I8 && engine != FTNN_ENGINE_MFMA_F4)) return 0;
+    if (rows <= 0 || K <= 0 || K > kMaxRowWords || (engine != FTNN_ENGINE_MFMA_I8 && engine != FTNN_ENGINE_MFMA_F4)) return 0;
     return mfma_fragment_bytes(engine == FTNN_ENGINE_MFMA_F4, rows, round4(K));
 }
 
 int ftnn_expand_rows(int engine, int ternary, const int64_t* d_rows, int rows, int K, void* d_out,
                      void* stream) {
-    if (rows <= 0 || K <= 0) return fail(FTNN_EINVAL, "non-positive dimension");
+    if (rows <= 0 || K <= 0 || K > kMaxRowWords) return fail(FTNN_EINVAL, "dimension non-positive or K too long");
     int rc = check_mfma_engine(engine, round4(K));
     if (rc != FTNN_OK) return rc;
     if (!d_rows || !d_out || !aligned16(d_rows) || !aligned16(d_out))
@@ -457,6 +468,7 @@ int ftnn_mm_expanded(int engine, int type, const void* d_a_exp, const void* d_b_
     if (type < kTNN || type > kBNN) return fail(FTNN_EINVAL, "unknown network type %d", type);
     if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0)
         return fail(FTNN_EINVAL, "non-positive GEMM dimension");
+    if (K > kMaxRowWords) return fail(FTNN_EINVAL, "K = %d words above the supported %d", K, kMaxRowWords);
     int rc = check_mfma_engine(engine, round4(K));
     if (rc != FTNN_OK) return rc;
     const int64_t M = (int64_t)N * OH * OW;
@@ -476,6 +488,7 @@ int ftnn_mm_engine(int engine, int type, const int64_t* d_a, const int64_t* d_b,
     if (type < kTNN || type > kBNN) return fail(FTNN_EINVAL, "unknown network type %d", type);
     if (N <= 0 || OH <= 0 || OW <= 0 || KN <= 0 || K <= 0)
         return fail(FTNN_EINVAL, "non-positive GEMM dimension");
+    if (K > kMaxRowWords) return fail(FTNN_EINVAL, "K = %d words above the supported %d", K, kMaxRowWords);
     const int64_t M = (int64_t)N * OH * OW;
     const int Kw = round4(K);
     if (engine == FTNN_ENGINE_AUTO) {
@@ -560,6 +573,7 @@ static int64_t prepared_bytes(int type, int C, int KN, int KH, int KW, int64_t* 
 
 int64_t ftnn_conv_weights_bytes(int type, int C, int KN, int KH, int KW) {
     if (type < kTNN || type > kBNN || C <= 0 || KN <= 0 || KH <= 0 || KW <= 0) return 0;
+    if (C > (1 << 30) || ((int64_t)C + 63) / 64 * KH * KW > kMaxRowWords) return 0;
     return prepared_bytes(type, C, KN, KH, KW, nullptr);
 }
 
@@ -567,6 +581,8 @@ int ftnn_conv_prepare_weights(int type, const int64_t* d_qw, int C, int KN, int 
                               void* stream) {
     if (type < kTNN || type > kBNN) return fail(FTNN_EINVAL, "unknown network type %d", type);
     if (C <= 0 || KN <= 0 || KH <= 0 || KW <= 0) return fail(FTNN_EINVAL, "non-positive dimension");
+    if (C > (1 << 30) || ((int64_t)C + 63) / 64 * KH * KW > kMaxRowWords)
+        return fail(FTNN_EINVAL, "more than %d words per weight row", kMaxRowWords);
     if (!d_qw || !d_prepared || !aligned16(d_qw) || !aligned16(d_prepared))
         return fail(FTNN_EINVAL, "null or misaligned device pointer");
     const bool wt = (type == kTNN || type == kBTN);
@@ -629,6 +645,8 @@ int ftnn_conv(int type, const float* d_x, const float* d_thr, const int64_t* d_q
 int ftnn_pack_weights(int ternary, const float* d_w, const float* d_thr, int KN, int C, int KH,
                       int KW, int64_t* d_out, void* stream) {
     if (KN <= 0 || C <= 0 || KH <= 0 || KW <= 0) return fail(FTNN_EINVAL, "non-positive dimension");
+    if (C > (1 << 30) || ((int64_t)C + 63) / 64 * KH * KW > kMaxRowWords)
+        return fail(FTNN_EINVAL, "more than %d words per weight row", kMaxRowWords);
     if (!d_w || !d_thr || !d_out) return fail(FTNN_EINVAL, "null device pointer");
     hipError_t e = launch_pack_weights(ternary != 0, d_w, d_thr, KN, C, KH, KW, d_out,
                                        (hipStream_t)stream);

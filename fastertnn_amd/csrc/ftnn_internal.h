@@ -197,6 +197,10 @@ __device__ __forceinline__ uint2 hand_over_block(const float (&r)[16], float alp
 // record a failure text for ftnn_last_error(); returns `code`
 int fail(int code, const char* fmt, ...);
 
+// shape and size-limit validation shared by every layer entry point; fills OH / OW; FTNN_OK or a recorded failure
+int check_conv_shape(int N, int C, int H, int W, int H_pad, int W_pad, int kH, int kW, int H_stride, int W_stride,
+                     int* OH, int* OW);
+
 // ---- pack_kernels.hip: launchers (arguments already validated) ----
 hipError_t launch_quantize_im2row(bool ternary, const float* d_x, const float* d_thr, int N, int C,
                                   int H, int W, int H_pad, int W_pad, int kH, int kW, int H_stride,

@@ -89,11 +89,16 @@ ftnn_net_t* ftnn_net_create(int batch, int n_layers, const ftnn_layer_t* layers)
     net->batch = batch;
     for (int i = 0; i < n_layers; i++) {
         const ftnn_layer_t& L = layers[i];
-        const bool ok = L.type >= kTNN && L.type <= kBNN && L.C > 0 && L.H > 0 && L.W > 0 && L.KN > 0 &&
-                        L.KH > 0 && L.KW > 0 && L.pad >= 0 && L.stride > 0 && L.H + 2 * L.pad >= L.KH &&
-                        L.W + 2 * L.pad >= L.KW && L.d_qw;
-        if (!ok) {
+        int oh = 0, ow = 0;
+        if (L.type < kTNN || L.type > kBNN || L.KN <= 0 || !L.d_qw) {
             fail(FTNN_EINVAL, "layer %d: bad description", i);
+            ftnn_net_destroy(net);
+            return nullptr;
+        }
+        // the same shape rules and size limits as a single layer call (the failure text is the check's)
+        if (check_conv_shape(batch, L.C, L.H, L.W, L.pad, L.pad, L.KH, L.KW, L.stride, L.stride, &oh, &ow) != FTNN_OK ||
+            ((int64_t)batch * oh * ow > 0x7fffff00LL &&
+             fail(FTNN_EINVAL, "layer %d: more than 2^31 output rows", i) != FTNN_OK)) {
             ftnn_net_destroy(net);
             return nullptr;
         }
@@ -107,15 +112,8 @@ ftnn_net_t* ftnn_net_create(int batch, int n_layers, const ftnn_layer_t* layers)
             }
         }
         net->layers.push_back(L);
-        net->OH.push_back(out_dim(L.H, L.pad, L.KH, L.stride));
-        net->OW.push_back(out_dim(L.W, L.pad, L.KW, L.stride));
-        // the same size limits as a single layer call
-        if (((int64_t)L.H + 2 * L.pad) * ((int64_t)L.W + 2 * L.pad) > 0x3ffffffLL ||
-            (int64_t)batch * net->OH[i] * net->OW[i] > 0x7fffff00LL) {
-            fail(FTNN_EINVAL, "layer %d: image plane above 2^26 pixels or more than 2^31 output rows", i);
-            ftnn_net_destroy(net);
-            return nullptr;
-        }
+        net->OH.push_back(oh);
+        net->OW.push_back(ow);
         net->out_elems = (int64_t)batch * L.KN * net->OH[i] * net->OW[i];
     }
     // engine of every layer, then the buffers the chain needs between them

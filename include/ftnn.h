@@ -114,9 +114,10 @@ FTNN_API float *mm_bnn(int64_t *a, int64_t *b, int N, int OH, int OW, int KN, in
 #define FTNN_ENOMEM (-3)  /* device or host allocation failed               */
 
 /* Size limits, all answered with FTNN_EINVAL: batch <= 65535; a padded image plane below
- * 2^26 pixels; at most 2^31-1 output rows (N*OH*OW); GEMM K below 2^18 words per plane on the
- * fp4 engine (exact fp32 accumulation).  Tensors themselves may exceed 2^32 elements: offsets
- * into them are 64-bit. */
+ * 2^26 pixels; at most 2^31-1 output rows (N*OH*OW); at most 2^24-4 words per plane of a row
+ * (GEMM K, ceil(C/64)*KH*KW of a layer: 32-bit sums), and below 2^18 on the fp4 engine (exact
+ * fp32 accumulation).  Tensors themselves may exceed 2^32 elements: offsets into them are
+ * 64-bit. */
 
 /* text of the last failure on the calling thread ("" if none) */
 FTNN_API const char *ftnn_last_error(void);

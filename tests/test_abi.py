@@ -172,3 +172,33 @@ def test_size_limits_need_no_device():
     big = lib.conv_scratch_bytes(0, 8, 1024, 56, 56, 1024, 3, 3, 1, 2)
     small = lib.conv_scratch_bytes(0, 8, 1024, 56, 56, 128, 3, 3, 1, 2)
     assert big > small > 0
+    # shape arithmetic that would overflow 32 bits is refused, not wrapped
+    assert lib.conv_scratch_bytes(0, 1, 1, 8, 8, 1, 3, 3, 2 ** 30, 1) == 0          # padding of 2^30
+    assert lib.conv_scratch_bytes(0, 1, 2 ** 31 - 1, 8, 8, 1, 3, 3, 1, 1) == 0      # channels near 2^31
+    assert lib.row_words(2 ** 31 - 1, 3, 3, True) == 0
+    assert lib.row_words(64 * (2 ** 24 - 4), 1, 1, False) == 2 ** 24 - 4            # the longest row
+    assert lib.row_words(64 * (2 ** 24 - 4) + 1, 1, 1, False) == 0
+    assert lib.mm_scratch_bytes(lib.ENGINE_MFMA_I8, 0, 256, 1, 1, 256, 2 ** 24) == 0
+
+
+def test_layer_chain_refuses_bad_descriptions_before_touching_the_device():
+    """ftnn_net_create validates every layer with the rules of a single layer call; nothing is allocated before"""
+    import ctypes
+    import fastertnn_amd.lib as lib
+
+    def create(batch, *shapes):
+        arr = (lib.LayerDesc * len(shapes))()
+        for d, (c, h, w, kn, kh, kw, pad, stride) in zip(arr, shapes):
+            d.type, d.C, d.H, d.W, d.KN, d.KH, d.KW, d.pad, d.stride = 0, c, h, w, kn, kh, kw, pad, stride
+            d.threshold, d.prelu_alpha, d.d_qw = 0.5, 0.5, ctypes.c_void_p(256)   # never read: validation fails first
+        return lib._L.ftnn_net_create(batch, len(shapes), arr), lib._L.ftnn_last_error().decode()
+
+    for batch, shapes, text in (
+            (1, [(64, 8, 8, 64, 3, 3, 2 ** 30, 1)], "2^26"),                       # padding that overflows 32 bits
+            (1, [(2 ** 31 - 1, 8, 8, 64, 3, 3, 1, 1)], "words per"),              # rows longer than 32-bit sums hold
+            (1, [(64, 8, 8, 64, 9, 9, 0, 1)], "larger than padded input"),
+            (70000, [(64, 8, 8, 64, 3, 3, 1, 1)], "batch"),
+            (1, [(64, 8, 8, 64, 3, 3, 1, 1), (32, 8, 8, 64, 3, 3, 1, 1)], "is not the output"),
+    ):
+        handle, err = create(batch, *shapes)
+        assert not handle and text in err, (shapes, err)
