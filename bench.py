@@ -286,7 +286,7 @@ RESNET18_LIKE = [  # (C, IH, IW, KN, KW, KH, pad, stride): stem, four stages wit
 ]
 
 
-def e2e_latency(torch, lib, batch, reps=10, cpu=True, typ=None):
+def e2e_latency(torch, lib, batch, reps=50, cpu=True, typ=None):
     """the ResNet-18-like TNN stack chained on the device (eager launches and HIP-graph replay), and
     (cpu=True) the same chain through the reference's tnns_conv on one host core"""
     import numpy as np
