@@ -7,6 +7,8 @@
 // layer's operand (P4) directly: the fp32 tensor in between (e.g. 103 MB after a batch-32 stem)
 // is neither written nor read, and the next layer needs no quantise launch.  The values compared
 // against the thresholds are the same fp32 numbers, so the chain's output is unchanged.
+#include <stdlib.h>
+
 #include <algorithm>
 #include <new>
 #include <vector>
@@ -14,15 +16,27 @@
 #include "../../include/ftnn.h"
 #include "ftnn_internal.h"
 
+// One share of the batch: a contiguous run of images with buffers of its own.  The images of a batch never meet
+// (every row of the GEMM belongs to one image), so a batch can run as two chains side by side on two streams: the
+// per-launch latency of one chain (a layer kernel here is a few microseconds long, a good part of it dispatch and
+// drain) then overlaps with the other chain's work.
+struct NetPart {
+    int first = 0, batch = 0;               // images [first, first + batch)
+    float* d_act[2] = {nullptr, nullptr};   // fp32 activations between layers that need them
+    void* d_p4[2] = {nullptr, nullptr};     // quantised input of the fp4 layers, by layer parity
+    void* d_scratch = nullptr;              // work space of the vector-ALU layers
+};
+
 struct ftnn_net {
     int batch = 0;
     std::vector<ftnn_layer_t> layers;
     std::vector<int> OH, OW;
     std::vector<float*> d_thr;       // per layer: batch copies of its threshold
     std::vector<void*> d_wf;         // per layer on the fp4 engine: its weights as matrix-core fragments
-    float* d_act[2] = {nullptr, nullptr};   // fp32 activations between layers that need them
-    void* d_p4[2] = {nullptr, nullptr};     // quantised input of the fp4 layers, by layer parity
-    void* d_scratch = nullptr;              // work space of the vector-ALU layers
+    std::vector<NetPart> parts;      // one, or two that run concurrently
+    hipStream_t side = nullptr;      // stream of the second part
+    hipEvent_t fork = nullptr, join = nullptr;
+    int64_t in_elems_per_image = 0, out_elems_per_image = 0;
     int64_t out_elems = 0;
     // recorded graph and what it was recorded for
     hipGraphExec_t exec = nullptr;
@@ -35,36 +49,65 @@ namespace {
 
 using namespace ftnn;
 
+// layer i of one part; `in` / `p4_ready` carry the part's state from layer to layer
+int enqueue_layer(ftnn_net* net, const NetPart& part, int i, const float*& in, bool& p4_ready, float* d_y,
+                  hipStream_t st) {
+    const int n = (int)net->layers.size();
+    const ftnn_layer_t& L = net->layers[i];
+    // the next layer takes a quantised hand-over if it is an fp4 layer that reads P4 (not a few-channel one)
+    const bool next_f4 = i + 1 < n && net->d_wf[i + 1] &&
+                         !dense_f4_applies(net->layers[i + 1].C, net->layers[i + 1].KH, net->layers[i + 1].KW);
+    QuantOut qo;
+    if (next_f4) {
+        const int nt = net->layers[i + 1].type;
+        qo.p4 = part.d_p4[(i + 1) & 1];
+        qo.thr = net->d_thr[i + 1];   // every entry holds the layer's threshold: any run of `batch` entries serves
+        qo.mode = (nt == kTNN || nt == kTBN) ? 1 : 2;
+    }
+    float* out = next_f4 ? nullptr : ((i == n - 1) ? d_y : part.d_act[i & 1]);
+    int rc;
+    if (net->d_wf[i])
+        rc = conv_f4_expanded(L.type, p4_ready ? nullptr : in, net->d_thr[i], net->d_wf[i], part.batch, L.C, L.H, L.W,
+                              L.KN, L.KH, L.KW, L.pad, L.pad, L.stride, L.stride, L.prelu_alpha, part.d_p4[i & 1], out,
+                              st, qo);
+    else
+        rc = conv_valu(L.type, in, net->d_thr[i], L.d_qw, part.batch, L.C, L.H, L.W, L.KN, L.KH, L.KW, L.pad, L.pad,
+                       L.stride, L.stride, L.prelu_alpha, part.d_scratch, out, st, qo, false);
+    p4_ready = next_f4;
+    in = out;
+    return rc;
+}
+
+// The whole batch: one chain on `st`, or two side by side (the second on the net's own stream, forked from and
+// joined back into `st` with events, which also holds under stream capture).  The launches of the two chains
+// alternate, so that both streams have work from the start.
 int enqueue_layers(ftnn_net* net, const float* d_x, float* d_y, hipStream_t st) {
     const int n = (int)net->layers.size();
-    const float* in = d_x;    // fp32 input of layer i (unused when p4_ready)
-    bool p4_ready = false;    // d_p4[i & 1] already holds layer i's quantised input
-    for (int i = 0; i < n; i++) {
-        const ftnn_layer_t& L = net->layers[i];
-        // the next layer takes a quantised hand-over if it is an fp4 layer that reads P4 (not a few-channel one)
-        const bool next_f4 = i + 1 < n && net->d_wf[i + 1] &&
-                             !dense_f4_applies(net->layers[i + 1].C, net->layers[i + 1].KH, net->layers[i + 1].KW);
-        QuantOut qo;
-        if (next_f4) {
-            const int nt = net->layers[i + 1].type;
-            qo.p4 = net->d_p4[(i + 1) & 1];
-            qo.thr = net->d_thr[i + 1];
-            qo.mode = (nt == kTNN || nt == kTBN) ? 1 : 2;
-        }
-        float* out = next_f4 ? nullptr : ((i == n - 1) ? d_y : net->d_act[i & 1]);
-        int rc;
-        if (net->d_wf[i])
-            rc = conv_f4_expanded(L.type, p4_ready ? nullptr : in, net->d_thr[i], net->d_wf[i], net->batch, L.C, L.H,
-                                  L.W, L.KN, L.KH, L.KW, L.pad, L.pad, L.stride, L.stride, L.prelu_alpha,
-                                  net->d_p4[i & 1], out, st, qo);
-        else
-            rc = conv_valu(L.type, in, net->d_thr[i], L.d_qw, net->batch, L.C, L.H, L.W, L.KN, L.KH, L.KW, L.pad,
-                           L.pad, L.stride, L.stride, L.prelu_alpha, net->d_scratch, out, st, qo, false);
-        if (rc != FTNN_OK) return rc;
-        p4_ready = next_f4;
-        in = out;
+    const size_t np = net->parts.size();
+    hipError_t e = hipSuccess;
+    if (np > 1) {
+        e = hipEventRecord(net->fork, st);
+        if (e == hipSuccess) e = hipStreamWaitEvent(net->side, net->fork, 0);
+        if (e != hipSuccess) return fail(FTNN_EHIP, "fork of the second chain: %s", hipGetErrorString(e));
     }
-    return FTNN_OK;
+    const float* in[2];
+    float* y[2];
+    bool p4_ready[2] = {false, false};
+    for (size_t p = 0; p < np; p++) {
+        in[p] = d_x + (size_t)net->parts[p].first * net->in_elems_per_image;
+        y[p] = d_y + (size_t)net->parts[p].first * net->out_elems_per_image;
+    }
+    int rc = FTNN_OK;
+    for (int i = 0; i < n && rc == FTNN_OK; i++)
+        for (size_t p = 0; p < np && rc == FTNN_OK; p++)
+            rc = enqueue_layer(net, net->parts[p], i, in[p], p4_ready[p], y[p], p == 0 ? st : net->side);
+    if (np > 1) {
+        // join even after a failure: a capture in progress must see the side stream return
+        e = hipEventRecord(net->join, net->side);
+        if (e == hipSuccess) e = hipStreamWaitEvent(st, net->join, 0);
+        if (rc == FTNN_OK && e != hipSuccess) rc = fail(FTNN_EHIP, "join of the second chain: %s", hipGetErrorString(e));
+    }
+    return rc;
 }
 
 void drop_graph(ftnn_net* net) {
@@ -116,32 +159,58 @@ ftnn_net_t* ftnn_net_create(int batch, int n_layers, const ftnn_layer_t* layers)
         net->OW.push_back(ow);
         net->out_elems = (int64_t)batch * L.KN * net->OH[i] * net->OW[i];
     }
-    // engine of every layer, then the buffers the chain needs between them
+    net->in_elems_per_image = (int64_t)layers[0].C * layers[0].H * layers[0].W;
+    net->out_elems_per_image = net->out_elems / batch;
+    // Two chains side by side from batch 48 on.  Measured on MI355X on a 19-layer ResNet-18-like stack (one chain /
+    // two): batch 48 0.218 / 0.195 ms, 64 0.240 / 0.214, 128 0.364 / 0.311, 256 0.609 / 0.519; at batch 32 the two
+    // chains' 38 launches take the host longer (0.19 ms) than the device needs for one chain (0.16 ms).
+    // FTNN_NET_PARTS = 1 / 2 overrides (tuning aid).
+    int nparts = batch >= 48 ? 2 : 1;
+    if (const char* env = getenv("FTNN_NET_PARTS")) nparts = atoi(env) >= 2 ? 2 : 1;
+    if (nparts > batch) nparts = 1;
+    net->parts.resize((size_t)nparts);
+    for (int p = 0, first = 0; p < nparts; p++) {
+        net->parts[(size_t)p].first = first;
+        net->parts[(size_t)p].batch = (batch - first + (nparts - p) - 1) / (nparts - p);
+        first += net->parts[(size_t)p].batch;
+    }
+    // engine of every layer (by the larger part: both parts must agree), then the buffers each part needs
+    const int pb = net->parts[0].batch;
     std::vector<char> f4((size_t)n_layers, 0);
     int64_t max_act = 0, max_scratch = 256, max_p4 = 0;
     for (int i = 0; i < n_layers; i++) {
         const ftnn_layer_t& L = layers[i];
-        f4[i] = ftnn_select_conv_engine(L.type, batch, L.C, L.H, L.W, L.KN, L.KH, L.KW, L.pad, L.pad, L.stride,
+        f4[i] = ftnn_select_conv_engine(L.type, pb, L.C, L.H, L.W, L.KN, L.KH, L.KW, L.pad, L.pad, L.stride,
                                         L.stride) == FTNN_ENGINE_MFMA_F4;
-        if (f4[i] && ((int64_t)batch * L.H * L.W * cpack_of(L.C) > 0x7fffffffLL ||
-                      (int64_t)batch * net->OH[i] * net->OW[i] * conv_f4_weight_words(L.C, L.KH, L.KW) > 0x7fffffffLL))
+        if (f4[i] && ((int64_t)pb * L.H * L.W * cpack_of(L.C) > 0x7fffffffLL ||
+                      (int64_t)pb * net->OH[i] * net->OW[i] * conv_f4_weight_words(L.C, L.KH, L.KW) > 0x7fffffffLL))
             f4[i] = 0;   // beyond the 32-bit pixel indices of the fp4 layer kernel: the vector-ALU layer takes it
-        if (f4[i]) {
-            max_p4 = std::max(max_p4, conv_f4_operand_bytes(batch, L.C, L.H, L.W, L.KH, L.KW, net->OH[i], net->OW[i], L.KN));
-            if (i > 0 && dense_f4_applies(L.C, L.KH, L.KW))   // its input arrives as fp32
-                max_act = std::max(max_act, (int64_t)batch * L.C * L.H * L.W);
-        } else {
-            max_scratch = std::max(max_scratch, ftnn_conv_scratch_bytes(L.type, batch, L.C, L.H, L.W, L.KN, L.KH, L.KW,
-                                                                        L.pad, L.pad, L.stride, L.stride));
-            if (i > 0)   // its input arrives as fp32
-                max_act = std::max(max_act, (int64_t)batch * L.C * L.H * L.W);
+        // sized for the larger part; a very large layer's operand region depends on the batch in steps (the
+        // im2row + GEMM form), so the smaller part is asked too
+        for (const NetPart& part : net->parts) {
+            if (f4[i])
+                max_p4 = std::max(max_p4, conv_f4_operand_bytes(part.batch, L.C, L.H, L.W, L.KH, L.KW, net->OH[i],
+                                                                net->OW[i], L.KN));
+            else
+                max_scratch = std::max(max_scratch, ftnn_conv_scratch_bytes(L.type, part.batch, L.C, L.H, L.W, L.KN, L.KH,
+                                                                            L.KW, L.pad, L.pad, L.stride, L.stride));
         }
+        // its input arrives as fp32 unless it is an fp4 layer that reads the previous layer's hand-over
+        if (i > 0 && (!f4[i] || dense_f4_applies(L.C, L.KH, L.KW)))
+            max_act = std::max(max_act, (int64_t)pb * L.C * L.H * L.W);
     }
-    bool good = hipMalloc(&net->d_scratch, (size_t)max_scratch) == hipSuccess;
-    for (int b = 0; b < 2 && good && max_act > 0; b++)
-        good = hipMalloc((void**)&net->d_act[b], (size_t)max_act * sizeof(float)) == hipSuccess;
-    for (int b = 0; b < 2 && good && max_p4 > 0; b++)
-        good = hipMalloc(&net->d_p4[b], (size_t)max_p4) == hipSuccess;
+    bool good = true;
+    for (NetPart& part : net->parts) {
+        good = good && hipMalloc(&part.d_scratch, (size_t)max_scratch) == hipSuccess;
+        for (int b = 0; b < 2 && good && max_act > 0; b++)
+            good = hipMalloc((void**)&part.d_act[b], (size_t)max_act * sizeof(float)) == hipSuccess;
+        for (int b = 0; b < 2 && good && max_p4 > 0; b++)
+            good = hipMalloc(&part.d_p4[b], (size_t)max_p4) == hipSuccess;
+    }
+    if (good && nparts > 1)
+        good = hipStreamCreateWithFlags(&net->side, hipStreamNonBlocking) == hipSuccess &&
+               hipEventCreateWithFlags(&net->fork, hipEventDisableTiming) == hipSuccess &&
+               hipEventCreateWithFlags(&net->join, hipEventDisableTiming) == hipSuccess;
     std::vector<float> host((size_t)batch);
     for (int i = 0; i < n_layers && good; i++) {
         float* d = nullptr;
@@ -186,11 +255,16 @@ void ftnn_net_destroy(ftnn_net_t* net) {
     for (float* p : net->d_thr) (void)hipFree(p);
     for (void* p : net->d_wf)
         if (p) (void)hipFree(p);
-    for (int b = 0; b < 2; b++)
-        if (net->d_act[b]) (void)hipFree(net->d_act[b]);
-    for (int b = 0; b < 2; b++)
-        if (net->d_p4[b]) (void)hipFree(net->d_p4[b]);
-    if (net->d_scratch) (void)hipFree(net->d_scratch);
+    for (NetPart& part : net->parts) {
+        for (int b = 0; b < 2; b++) {
+            if (part.d_act[b]) (void)hipFree(part.d_act[b]);
+            if (part.d_p4[b]) (void)hipFree(part.d_p4[b]);
+        }
+        if (part.d_scratch) (void)hipFree(part.d_scratch);
+    }
+    if (net->fork) (void)hipEventDestroy(net->fork);
+    if (net->join) (void)hipEventDestroy(net->join);
+    if (net->side) (void)hipStreamDestroy(net->side);
     delete net;
 }
 

@@ -250,7 +250,10 @@ FTNN_API int ftnn_conv_prepared(int type, const float *d_x, const float *d_thr, 
  * reference's chain of tnns_conv calls returns, bit for bit.  All device memory (activation
  * and operand buffers, work space, per-layer threshold arrays, the weights in engine form) is
  * allocated by ftnn_net_create; a run allocates nothing.  Packed weights stay the caller's and
- * must outlive the net.
+ * must outlive the net.  From batch 48 on a net runs the two halves of its batch as two chains
+ * side by side (the second on a stream of its own, forked from and joined back into the
+ * caller's stream inside ftnn_net_run, also under graph capture): the images of a batch never
+ * meet, and the launch latencies of one chain overlap with the other's work.
  */
 typedef struct ftnn_layer {
     int type;             /* TNN / TBN / BTN / BNN                               */

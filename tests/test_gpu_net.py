@@ -115,6 +115,36 @@ def test_other_chains_match_the_oracle(hip, oracle, which):
     net.close()
 
 
+@pytest.mark.parametrize("which,batch", [(1, 2), (1, 5), (2, 3), (3, 17)])
+def test_batch_split_over_two_concurrent_chains(hip, oracle, monkeypatch, which, batch):
+    """a net may run its batch as two chains side by side on two streams (by default from batch 16 on; forced
+    here for small and odd batches): same bits as one chain and as the oracle, eager and as replayed graph, over
+    repeated runs that reuse the parts' buffers"""
+    import torch
+    stack = {1: STACK, 2: STACK2, 3: STACK3}[which]
+    c, ih, iw = stack[0][1][:3]
+    x = synth.normal(40 + which, (batch, c, ih, iw))
+    xd = torch.from_numpy(x).cuda()
+    outs = {}
+    for parts in ("1", "2"):
+        monkeypatch.setenv("FTNN_NET_PARTS", parts)
+        net, host = build(hip, oracle, batch, stack)
+        s = torch.cuda.Stream()
+        with torch.cuda.stream(s):
+            for rep in range(3):
+                for graph in (False, True):
+                    out = torch.full(net.out_shape, -1.0, device="cuda")
+                    net.run(xd, out=out, graph=graph)
+                    s.synchronize()
+                    outs.setdefault(parts, out.cpu().numpy())
+                    assert out.cpu().numpy().tobytes() == outs[parts].tobytes(), (parts, rep, graph)
+                    (torch.ones(1000, device="cuda") * rep).sum().item()
+        net.close()
+    want = oracle_chain(oracle, host, x)
+    assert outs["1"].tobytes() == want.tobytes()
+    assert outs["2"].tobytes() == want.tobytes()
+
+
 def test_chain_rejects_mismatched_layers(hip, oracle):
     import torch
     qw = torch.zeros(64 * 2 * 4, dtype=torch.int64, device="cuda")
