@@ -81,3 +81,21 @@ def test_hip_layer_equals_the_reference_baseline_build(hip, oracle, reference_ba
         qw2 = oracle.pack_weights(L["w"], L["wthr"], wt)
         got = hip.host_conv(typ, L["x"], L["thr"], qw2, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], L["alpha"])
         assert got.tobytes() == want.tobytes()
+
+
+def test_large_buffers_through_the_host_entry_points(hip, oracle):
+    """inputs and results of 20 MB: the host entry points move them through their ring of pinned chunks (several
+    trips round the ring, a partial last chunk) with the copy threads; twice, so that the ring is reused"""
+    shape = (64, 100, 101, 64, 3, 3, 1, 1)
+    L = make_layer(TNN, shape, 8, seed=4242)
+    assert L["x"].nbytes > 16 << 20
+    qw = oracle.pack_weights(L["w"], L["wthr"], True)
+    want = oracle.conv(TNN, L["x"], L["thr"], qw, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], L["alpha"])
+    for rep in range(2):
+        got = hip.host_conv(TNN, L["x"], L["thr"], qw, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], L["alpha"])
+        assert got.nbytes > 16 << 20 and got.tobytes() == want.tobytes(), rep
+    rows_o = oracle.quantize_im2row(L["x"], L["thr"], 3, 3, 1, 1, True)
+    rows_h = hip.host_quantize_im2row(L["x"], L["thr"], 3, 3, 1, 1, True)
+    assert rows_h.nbytes > 12 << 20 and np.array_equal(rows_h, rows_o)
+    y_h = hip.host_mm(TNN, rows_o, qw, 8, 100, 101, 64, 9, L["alpha"], 0)
+    assert y_h.tobytes() == want.tobytes()
