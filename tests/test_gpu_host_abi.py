@@ -99,3 +99,36 @@ def test_large_buffers_through_the_host_entry_points(hip, oracle):
     assert rows_h.nbytes > 12 << 20 and np.array_equal(rows_h, rows_o)
     y_h = hip.host_mm(TNN, rows_o, qw, 8, 100, 101, 64, 9, L["alpha"], 0)
     assert y_h.tobytes() == want.tobytes()
+
+
+_CHILD = r"""
+import sys
+import numpy as np, torch
+sys.path.insert(0, sys.argv[1])
+import fastertnn_amd.lib as hip
+from fastertnn_amd import TNN
+from tests.cases import make_layer
+L = make_layer(TNN, (64, 100, 101, 64, 3, 3, 1, 1), 8, seed=4242)
+qw = hip.pack_weights(torch.from_numpy(L["w"]).cuda(), torch.from_numpy(L["wthr"]).cuda(), True)
+want = hip.conv(TNN, torch.from_numpy(L["x"]).cuda(), torch.from_numpy(L["thr"]).cuda(), qw, L["kn"], 3, 3, 1, 1,
+                L["alpha"]).cpu().numpy()
+for rep in range(2):
+    got = hip.host_conv(TNN, L["x"], L["thr"], qw.cpu().numpy(), L["kn"], 3, 3, 1, 1, L["alpha"])
+    assert got.tobytes() == want.tobytes(), rep
+print("child ok")
+"""
+
+
+@pytest.mark.parametrize("threads", ["1", "3"])
+def test_host_copies_with_other_thread_counts(threads):
+    """the copy threads of the host entry points are a per-process choice (CPU affinity, or FTNN_HOST_COPY_THREADS):
+    one thread takes the runtime's plain copies, three an odd split of every chunk; a child process each, checked
+    against the device-resident call"""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, FTNN_HOST_COPY_THREADS=threads)
+    print("case host copy threads", threads, flush=True)
+    r = subprocess.run([sys.executable, "-c", _CHILD, root], env=env, capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0 and "child ok" in r.stdout, r.stdout[-1500:] + r.stderr[-1500:]
