@@ -10,7 +10,9 @@
 #include <algorithm>
 #include <condition_variable>
 #include <mutex>
+#include <system_error>
 #include <thread>
+#include <vector>
 
 #include "../../include/ftnn.h"
 #include "ftnn_internal.h"
@@ -149,8 +151,17 @@ private:
         if (sched_getaffinity(0, sizeof(set), &set) == 0) cores = CPU_COUNT(&set);
         int threads = std::min(cores, 8);
         if (const char* env = getenv("FTNN_HOST_COPY_THREADS")) threads = std::max(1, std::min(atoi(env), 16));   // tuning aid
-        workers_ = threads - 1;   // a caller pinned to one core (the reference's Makefile) copies alone
-        for (int t = 0; t < workers_; t++) std::thread([this, t] { run(t); }).detach();
+        const int wanted = threads - 1;   // a caller pinned to one core (the reference's Makefile) copies alone
+        // workers_ is final before the first worker runs: a slice's bounds depend on it
+        std::vector<std::thread> started;
+        try {
+            for (int t = 0; t < wanted; t++) started.emplace_back([this, t] { run(t); });
+        } catch (const std::system_error&) {   // no more threads to be had: go on with those that started
+        }
+        std::unique_lock<std::mutex> lock(m_);
+        workers_ = (int)started.size();
+        lock.unlock();
+        for (std::thread& th : started) th.detach();
     }
     void slice(int t) {
         const size_t parts = (size_t)workers_ + 1;
