@@ -33,6 +33,7 @@ struct ftnn_net {
     std::vector<int> OH, OW;
     std::vector<float*> d_thr;       // per layer: batch copies of its threshold
     std::vector<void*> d_wf;         // per layer on the fp4 engine: its weights as matrix-core fragments
+    std::vector<char> rereads;       // per layer: its input is the leading part of the previous layer's fp32 output
     std::vector<NetPart> parts;      // one, or two that run concurrently
     hipStream_t side = nullptr;      // stream of the second part
     hipEvent_t fork = nullptr, join = nullptr;
@@ -55,7 +56,7 @@ int enqueue_layer(ftnn_net* net, const NetPart& part, int i, const float*& in, b
     const int n = (int)net->layers.size();
     const ftnn_layer_t& L = net->layers[i];
     // the next layer takes a quantised hand-over if it is an fp4 layer that reads P4 (not a few-channel one)
-    const bool next_f4 = i + 1 < n && net->d_wf[i + 1] &&
+    const bool next_f4 = i + 1 < n && net->d_wf[i + 1] && !net->rereads[i + 1] &&
                          !dense_f4_applies(net->layers[i + 1].C, net->layers[i + 1].KH, net->layers[i + 1].KW);
     QuantOut qo;
     if (next_f4) {
@@ -120,6 +121,14 @@ void drop_graph(ftnn_net* net) {
 extern "C" {
 
 ftnn_net_t* ftnn_net_create(int batch, int n_layers, const ftnn_layer_t* layers) {
+    return ftnn_net_create_ex(batch, n_layers, layers, 0);
+}
+
+ftnn_net_t* ftnn_net_create_ex(int batch, int n_layers, const ftnn_layer_t* layers, int flags) {
+    if (flags & ~FTNN_NET_REREAD_PREFIX) {
+        fail(FTNN_EINVAL, "unknown flags 0x%x", flags);
+        return nullptr;
+    }
     if (batch <= 0 || batch > 65535 || n_layers <= 0 || !layers) {
         fail(FTNN_EINVAL, "bad batch or layer count");
         return nullptr;
@@ -145,15 +154,23 @@ ftnn_net_t* ftnn_net_create(int batch, int n_layers, const ftnn_layer_t* layers)
             ftnn_net_destroy(net);
             return nullptr;
         }
+        char reread = 0;
         if (i > 0) {
             const ftnn_layer_t& P = layers[i - 1];
             if (L.C != P.KN || L.H != net->OH[i - 1] || L.W != net->OW[i - 1]) {
-                fail(FTNN_EINVAL, "layer %d: input %dx%dx%d is not the output %dx%dx%d of layer %d", i, L.C, L.H,
-                     L.W, P.KN, net->OH[i - 1], net->OW[i - 1], i - 1);
-                ftnn_net_destroy(net);
-                return nullptr;
+                // the reference's e2e driver hands the previous output buffer on whatever the next table row says
+                // (src/timing_layers.c:187-200): the next layer then reads the buffer's leading floats as its NCHW input
+                const int64_t have = (int64_t)P.KN * net->OH[i - 1] * net->OW[i - 1], want = (int64_t)L.C * L.H * L.W;
+                if (!(flags & FTNN_NET_REREAD_PREFIX) || want > have) {
+                    fail(FTNN_EINVAL, "layer %d: input %dx%dx%d is not the output %dx%dx%d of layer %d", i, L.C, L.H,
+                         L.W, P.KN, net->OH[i - 1], net->OW[i - 1], i - 1);
+                    ftnn_net_destroy(net);
+                    return nullptr;
+                }
+                reread = 1;
             }
         }
+        net->rereads.push_back(reread);
         net->layers.push_back(L);
         net->OH.push_back(oh);
         net->OW.push_back(ow);
@@ -168,6 +185,8 @@ ftnn_net_t* ftnn_net_create(int batch, int n_layers, const ftnn_layer_t* layers)
     int nparts = batch >= 48 ? 2 : 1;
     if (const char* env = getenv("FTNN_NET_PARTS")) nparts = atoi(env) >= 2 ? 2 : 1;
     if (nparts > batch) nparts = 1;
+    for (char r : net->rereads)
+        if (r) nparts = 1;   // such a layer's input runs across the images of the previous output
     net->parts.resize((size_t)nparts);
     for (int p = 0, first = 0; p < nparts; p++) {
         net->parts[(size_t)p].first = first;
@@ -198,6 +217,8 @@ ftnn_net_t* ftnn_net_create(int batch, int n_layers, const ftnn_layer_t* layers)
         // its input arrives as fp32 unless it is an fp4 layer that reads the previous layer's hand-over
         if (i > 0 && (!f4[i] || dense_f4_applies(L.C, L.KH, L.KW)))
             max_act = std::max(max_act, (int64_t)pb * L.C * L.H * L.W);
+        if (i > 0 && net->rereads[i])   // the previous layer writes its whole fp32 output, this one reads the start of it
+            max_act = std::max(max_act, (int64_t)pb * layers[i - 1].KN * net->OH[i - 1] * net->OW[i - 1]);
     }
     bool good = true;
     for (NetPart& part : net->parts) {

@@ -67,7 +67,7 @@ EXPORTS = ("tnns_conv", "tnns_gemm", "t2r_p2_opt", "b2r", "mm_tnn", "mm_tbn", "m
            "ftnn_pack_weights", "ftnn_pack_gemm_operand", "ftnn_select_engine", "ftnn_mm_scratch_bytes",
            "ftnn_mm_engine", "ftnn_expand_bytes", "ftnn_expand_rows", "ftnn_mm_expanded",
            "ftnn_conv_scratch_bytes", "ftnn_conv_engine", "ftnn_select_conv_engine",
-           "ftnn_conv_weights_bytes", "ftnn_conv_prepare_weights", "ftnn_conv_prepared", "ftnn_net_create", "ftnn_net_destroy", "ftnn_net_output_elems", "ftnn_net_run")
+           "ftnn_conv_weights_bytes", "ftnn_conv_prepare_weights", "ftnn_conv_prepared", "ftnn_net_create", "ftnn_net_create_ex", "ftnn_net_destroy", "ftnn_net_output_elems", "ftnn_net_run")
 
 ENGINE_AUTO, ENGINE_VALU, ENGINE_MFMA_I8, ENGINE_MFMA_F4 = 0, 1, 2, 3
 ENGINE_NAMES = {ENGINE_VALU: "valu", ENGINE_MFMA_I8: "mfma_i8", ENGINE_MFMA_F4: "mfma_f4"}
@@ -264,6 +264,9 @@ class LayerDesc(C.Structure):
 
 _L.ftnn_net_create.restype = _vp
 _L.ftnn_net_create.argtypes = [C.c_int, C.c_int, C.POINTER(LayerDesc)]
+_L.ftnn_net_create_ex.restype = _vp
+_L.ftnn_net_create_ex.argtypes = [C.c_int, C.c_int, C.POINTER(LayerDesc), C.c_int]
+NET_REREAD_PREFIX = 1
 _L.ftnn_net_destroy.restype = None
 _L.ftnn_net_destroy.argtypes = [_vp]
 _L.ftnn_net_output_elems.restype = C.c_int64
@@ -276,7 +279,7 @@ class Net:
     `layers` is a list of dicts with keys type, shape (C, IH, IW, KN, KW, KH, pad, stride),
     threshold, alpha, qw (packed weights, int64 CUDA tensor, kept alive here)."""
 
-    def __init__(self, batch, layers):
+    def __init__(self, batch, layers, flags=0):
         self.batch = batch
         self._weights = [l["qw"] for l in layers]
         arr = (LayerDesc * len(layers))()
@@ -284,7 +287,7 @@ class Net:
             c, ih, iw, kn, kw, kh, pad, stride = l["shape"]
             d.type, d.C, d.H, d.W, d.KN, d.KH, d.KW, d.pad, d.stride = l["type"], c, ih, iw, kn, kh, kw, pad, stride
             d.threshold, d.prelu_alpha, d.d_qw = l["threshold"], l["alpha"], _dev(l["qw"])
-        self._h = _L.ftnn_net_create(batch, len(layers), arr)
+        self._h = _L.ftnn_net_create_ex(batch, len(layers), arr, flags) if flags else _L.ftnn_net_create(batch, len(layers), arr)
         if not self._h:
             raise FtnnError(_L.ftnn_last_error().decode())
         c, ih, iw, kn, kw, kh, pad, stride = layers[-1]["shape"]

@@ -270,6 +270,14 @@ typedef struct ftnn_net ftnn_net_t;
 /* NULL on failure (ftnn_last_error() says why): every layer's input must be the previous
  * layer's output shape */
 FTNN_API ftnn_net_t *ftnn_net_create(int batch, int n_layers, const ftnn_layer_t *layers);
+/* The same with flags.  FTNN_NET_REREAD_PREFIX accepts a layer whose input shape is not the
+ * previous layer's output shape, provided it is no larger: the layer then takes the leading
+ * N*C*H*W floats of the previous fp32 output as its NCHW input.  That is what the reference's e2e
+ * driver does on its tables that leave out the pooling layers (ResNet-34, VGG-16, VGG-19 of
+ * include/timing/shapes_e2e.h: src/timing_layers.c:187-200 hands the output buffer on whatever
+ * the next row says); without the flag such a table is refused. */
+#define FTNN_NET_REREAD_PREFIX 1
+FTNN_API ftnn_net_t *ftnn_net_create_ex(int batch, int n_layers, const ftnn_layer_t *layers, int flags);
 FTNN_API void ftnn_net_destroy(ftnn_net_t *net);
 /* elements of the final output (batch * KN * OH * OW of the last layer) */
 FTNN_API int64_t ftnn_net_output_elems(const ftnn_net_t *net);

@@ -202,3 +202,14 @@ def test_layer_chain_refuses_bad_descriptions_before_touching_the_device():
     ):
         handle, err = create(batch, *shapes)
         assert not handle and text in err, (shapes, err)
+
+
+def test_layer_chain_refuses_unknown_flags():
+    import ctypes
+    import fastertnn_amd.lib as lib
+    arr = (lib.LayerDesc * 1)()
+    d = arr[0]
+    d.type, d.C, d.H, d.W, d.KN, d.KH, d.KW, d.pad, d.stride = 0, 64, 8, 8, 64, 3, 3, 1, 1
+    d.threshold, d.prelu_alpha, d.d_qw = 0.5, 0.5, ctypes.c_void_p(256)
+    assert not lib._L.ftnn_net_create_ex(1, 1, arr, 6)
+    assert "flags" in lib._L.ftnn_last_error().decode()
