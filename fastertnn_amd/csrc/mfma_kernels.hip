@@ -342,10 +342,16 @@ struct ConvFrag {
 // All three are compile-time so that the per-element epilogue carries no selects for them.
 // The unsplit hand-over variants are the ones launched with several thousand wavefronts (stems,
 // first stages): they are asked to fit three wavefronts per SIMD, which they do without scratch.
-template <bool ABIN, bool FORM0, int QMODE, int S, int NB>
+// BUF (ternary activations only): fragments arrive through buffer loads.  Their offsets are 32-bit, the weight
+// fragment of a word is addressed by a scalar offset alone, and an offset beyond the buffer returns zeros, which is
+// what a tap outside the image must contribute: no select on the loaded data, a third of the K loop's vector
+// instructions gone.  Needs both operands below 4 GiB (p4_bytes, wf_bytes: the sizes the descriptors announce).
+template <bool ABIN, bool FORM0, int QMODE, int S, int NB, bool BUF>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && QMODE != 0) ? 3 : 1, 8))) void k_conv_f4(const uint4* __restrict__ P4, const uint4* __restrict__ Wf,
                                                  float* __restrict__ Y, int M, int KN, int OHW, int KB,
-                                                 int bias, float alpha, FastDiv dOHW, ConvGeom cg, QuantOut qo) {
+                                                 int bias, float alpha, FastDiv dOHW, ConvGeom cg, QuantOut qo,
+                                                 uint32_t p4_bytes, uint32_t wf_bytes) {
+    static_assert(!(BUF && ABIN), "binary activations pad with +1, not with the zeros an out-of-range buffer load returns");
     // NB register sets of fragments: NB - 1 steps of loads in flight
     constexpr int WPB = 4;                // wavefronts per workgroup (single-wavefront workgroups for S = 1
                                           // measured slower: neighbours no longer share weight fragments in L1)
@@ -401,18 +407,48 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
     auto ld16 = [](v4i& dst, const uint4* src) {
         asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(dst) : "v"(src) : "memory");
     };
+    // buffer descriptors (base, 48-bit; stride 0; bytes; raw 32-bit data format) and this lane's fixed offsets
+    v4i rsrc_x = {0, 0, 0, 0}, rsrc_w = {0, 0, 0, 0};
+    uint32_t wofs[2] = {0u, 0u};
+    if constexpr (BUF) {
+        const uint64_t px = reinterpret_cast<uint64_t>(P4), pw = reinterpret_cast<uint64_t>(Wf);
+        rsrc_x = v4i{__builtin_amdgcn_readfirstlane((int)(uint32_t)px), __builtin_amdgcn_readfirstlane((int)((px >> 32) & 0xffffu)),
+                     __builtin_amdgcn_readfirstlane((int)p4_bytes), 0x00020000};
+        rsrc_w = v4i{__builtin_amdgcn_readfirstlane((int)(uint32_t)pw), __builtin_amdgcn_readfirstlane((int)((pw >> 32) & 0xffffu)),
+                     __builtin_amdgcn_readfirstlane((int)wf_bytes), 0x00020000};
+#pragma unroll
+        for (int a = 0; a < 2; a++) wofs[a] = ((uint32_t)min(kn0 / 32 + a, rbmax) * (uint32_t)KB * 64u + (uint32_t)lane) * 16u;
+    }
+    auto ldbuf = [](v4i& dst, uint32_t voff, const v4i& rsrc, uint32_t soff) {
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(dst) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+    };
     auto load = [&](int w, ConvFrag& f) {   // w is wave-uniform
         const int tap = (int)fastdiv((uint32_t)w, cg.dCP), ic = w - tap * cg.CP;
         const int kh = (int)fastdiv((uint32_t)tap, cg.dKW), kw = tap - kh * cg.KW;
+        if constexpr (BUF) {
+            const uint32_t wsoff = (uint32_t)__builtin_amdgcn_readfirstlane(w) * 1024u;
 #pragma unroll
-        for (int a = 0; a < 2; a++) ld16(f.w[a], wb[a] + (size_t)w * 64);
+            for (int a = 0; a < 2; a++) ldbuf(f.w[a], wofs[a], rsrc_w, wsoff);
+            const uint32_t icoff = (uint32_t)__builtin_amdgcn_readfirstlane(ic * HWin);
 #pragma unroll
-        for (int b = 0; b < 2; b++) {
-            const int ih = ih0[b] + kh, iw = iw0[b] + kw;
-            const bool in = (unsigned)ih < (unsigned)cg.H && (unsigned)iw < (unsigned)cg.W;
-            const size_t o = (size_t)(pb[b] + (uint32_t)(ic * HWin + (in ? ih * cg.W + iw : 0))) * 2 + h;
-            ld16(f.x[b], P4 + o);
-            f.in[b] = in;
+            for (int b = 0; b < 2; b++) {
+                const int ih = ih0[b] + kh, iw = iw0[b] + kw;
+                const bool in = (unsigned)ih < (unsigned)cg.H && (unsigned)iw < (unsigned)cg.W;
+                const uint32_t o = ((pb[b] + icoff + (uint32_t)(ih * cg.W + iw)) * 2u + (uint32_t)h) * 16u;
+                ldbuf(f.x[b], in ? o : 0xffffff00u, rsrc_x, 0u);   // beyond p4_bytes: the load returns zeros
+                f.in[b] = true;
+            }
+        } else {
+#pragma unroll
+            for (int a = 0; a < 2; a++) ld16(f.w[a], wb[a] + (size_t)w * 64);
+#pragma unroll
+            for (int b = 0; b < 2; b++) {
+                const int ih = ih0[b] + kh, iw = iw0[b] + kw;
+                const bool in = (unsigned)ih < (unsigned)cg.H && (unsigned)iw < (unsigned)cg.W;
+                const size_t o = (size_t)(pb[b] + (uint32_t)(ic * HWin + (in ? ih * cg.W + iw : 0))) * 2 + h;
+                ld16(f.x[b], P4 + o);
+                f.in[b] = in;
+            }
         }
     };
     auto arrive = [](ConvFrag& f, auto outstanding) {
@@ -426,7 +462,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
 #pragma unroll
         for (int b = 0; b < 2; b++) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) x[b][i] = f.in[b] ? f.x[b][i] : (int)fillv;
+            for (int i = 0; i < 4; i++) x[b][i] = (BUF || f.in[b]) ? f.x[b][i] : (int)fillv;
 #pragma unroll
             for (int i = 4; i < 8; i++) x[b][i] = 0;
         }
@@ -799,15 +835,40 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
         hipLaunchKernelGGL(kern, grid, dim3(64 * wpb), 0, st, P4, Wf, d_y, (int)M, KN, OHW, KB, bias, alpha, dOHW, cg, qo);
         return hipGetLastError();
     };
+    // the 64 x 64 kernel takes two sizes more (its buffer-load variant announces them in its descriptors)
+    const int64_t p4_bytes = (int64_t)N * cg.CP * cg.H * cg.W * 32, wf_bytes = (int64_t)((KN + 31) / 32) * KB * 1024;
+    static const bool no_buf = getenv("FTNN_CONV_NO_BUFFER_LOADS") != nullptr;   // tuning aid
+    const bool buf = !no_buf && p4_bytes <= 0xf0000000LL && wf_bytes <= 0xf0000000LL;
+    auto launch64 = [&](auto variant) -> hipError_t {
+        constexpr auto kern = decltype(variant)::value;
+        static const hipError_t sound = []() {
+            hipFuncAttributes attr;
+            hipError_t e = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(kern));
+            if (e == hipSuccess && attr.localSizeBytes != 0) e = hipErrorLaunchFailure;
+            return e;
+        }();
+        if (sound != hipSuccess) return sound;
+        hipLaunchKernelGGL(kern, grid, dim3(64 * wpb), 0, st, P4, Wf, d_y, (int)M, KN, OHW, KB, bias, alpha, dOHW, cg, qo,
+                           (uint32_t)std::min<int64_t>(p4_bytes, 0xffffffffLL), (uint32_t)std::min<int64_t>(wf_bytes, 0xffffffffLL));
+        return hipGetLastError();
+    };
+    auto by_buf = [&](auto abin, auto form0, auto qmode, auto sp) -> hipError_t {
+        constexpr bool A = decltype(abin)::value, F = decltype(form0)::value;
+        constexpr int Q = decltype(qmode)::value, SP = decltype(sp)::value;
+        if constexpr (!A) {
+            if (buf) return launch64(std::integral_constant<decltype(&k_conv_f4<A, F, Q, SP, 3, true>), &k_conv_f4<A, F, Q, SP, 3, true>>{});
+        }
+        return launch64(std::integral_constant<decltype(&k_conv_f4<A, F, Q, SP, 3, false>), &k_conv_f4<A, F, Q, SP, 3, false>>{});
+    };
     // kernel variant: activation kind and PReLU form follow the type, then hand-over mode and split
     auto by_split = [&](auto abin, auto form0, auto qmode) -> hipError_t {
         constexpr bool A = decltype(abin)::value, F = decltype(form0)::value;
         constexpr int Q = decltype(qmode)::value;
         if (small) return launch(std::integral_constant<decltype(&k_conv_f4_small<A, F, Q>), &k_conv_f4_small<A, F, Q>>{});
         // three register sets: deeper prefetch measured no faster at any layer size
-        if (split == 1) return launch(std::integral_constant<decltype(&k_conv_f4<A, F, Q, 1, 3>), &k_conv_f4<A, F, Q, 1, 3>>{});
-        if (split == 2) return launch(std::integral_constant<decltype(&k_conv_f4<A, F, Q, 2, 3>), &k_conv_f4<A, F, Q, 2, 3>>{});
-        if (split == 4) return launch(std::integral_constant<decltype(&k_conv_f4<A, F, Q, 4, 3>), &k_conv_f4<A, F, Q, 4, 3>>{});
+        if (split == 1) return by_buf(abin, form0, qmode, std::integral_constant<int, 1>{});
+        if (split == 2) return by_buf(abin, form0, qmode, std::integral_constant<int, 2>{});
+        if (split == 4) return by_buf(abin, form0, qmode, std::integral_constant<int, 4>{});
         return hipErrorInvalidValue;
     };
     auto by_mode = [&](auto abin, auto form0) -> hipError_t {
