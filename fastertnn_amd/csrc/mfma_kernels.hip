@@ -409,7 +409,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
     };
     // buffer descriptors (base, 48-bit; stride 0; bytes; raw 32-bit data format) and this lane's fixed offsets
     v4i rsrc_x = {0, 0, 0, 0}, rsrc_w = {0, 0, 0, 0};
-    uint32_t wofs[2] = {0u, 0u};
+    uint32_t wofs[2] = {0u, 0u}, xofs[2] = {0u, 0u};
     if constexpr (BUF) {
         const uint64_t px = reinterpret_cast<uint64_t>(P4), pw = reinterpret_cast<uint64_t>(Wf);
         rsrc_x = v4i{__builtin_amdgcn_readfirstlane((int)(uint32_t)px), __builtin_amdgcn_readfirstlane((int)((px >> 32) & 0xffffu)),
@@ -418,6 +418,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
                      __builtin_amdgcn_readfirstlane((int)wf_bytes), 0x00020000};
 #pragma unroll
         for (int a = 0; a < 2; a++) wofs[a] = ((uint32_t)min(kn0 / 32 + a, rbmax) * (uint32_t)KB * 64u + (uint32_t)lane) * 16u;
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+            xofs[b] = ((pb[b] + (uint32_t)(ih0[b] * cg.W + iw0[b])) * 2u + (uint32_t)h) * 16u;
     }
     auto ldbuf = [](v4i& dst, uint32_t voff, const v4i& rsrc, uint32_t soff) {
         asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(dst) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
@@ -429,13 +432,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
             const uint32_t wsoff = (uint32_t)__builtin_amdgcn_readfirstlane(w) * 1024u;
 #pragma unroll
             for (int a = 0; a < 2; a++) ldbuf(f.w[a], wofs[a], rsrc_w, wsoff);
-            const uint32_t icoff = (uint32_t)__builtin_amdgcn_readfirstlane(ic * HWin);
+            // byte offset of the record = this lane's part (xofs, fixed) + the word's part (scalar); the sum wraps
+            // to the right value whenever the tap lies inside the image
+            const uint32_t tapoff = (uint32_t)__builtin_amdgcn_readfirstlane((ic * HWin + kh * cg.W + kw) * 32);
 #pragma unroll
             for (int b = 0; b < 2; b++) {
                 const int ih = ih0[b] + kh, iw = iw0[b] + kw;
                 const bool in = (unsigned)ih < (unsigned)cg.H && (unsigned)iw < (unsigned)cg.W;
-                const uint32_t o = ((pb[b] + icoff + (uint32_t)(ih * cg.W + iw)) * 2u + (uint32_t)h) * 16u;
-                ldbuf(f.x[b], in ? o : 0xffffff00u, rsrc_x, 0u);   // beyond p4_bytes: the load returns zeros
+                ldbuf(f.x[b], in ? xofs[b] + tapoff : 0xffffff00u, rsrc_x, 0u);   // beyond p4_bytes: the load returns zeros
                 f.in[b] = true;
             }
         } else {
