@@ -596,10 +596,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
 // one activation fragment per word), wavefronts 1..3 hand their partial block over through LDS and wavefront 0
 // finishes it.  Kernel tiles come in pairs under the hand-over (a pixel's 64-channel word is written by two
 // workgroups, 16 bytes each; a tile past KN writes padding lanes).
-template <bool ABIN, bool FORM0, int QMODE>
+// BUF: fragments through buffer loads, as in k_conv_f4.
+template <bool ABIN, bool FORM0, int QMODE, bool BUF>
 __global__ __launch_bounds__(256) void k_conv_f4_small(const uint4* __restrict__ P4, const uint4* __restrict__ Wf,
                                                        float* __restrict__ Y, int M, int KN, int OHW, int KB, int bias,
-                                                       float alpha, FastDiv dOHW, ConvGeom cg, QuantOut qo) {
+                                                       float alpha, FastDiv dOHW, ConvGeom cg, QuantOut qo,
+                                                       uint32_t p4_bytes, uint32_t wf_bytes) {
+    static_assert(!(BUF && ABIN), "binary activations pad with +1");
     constexpr int S = 4, NB = 3;
     __shared__ float4 red[3 * 4 * 64];   // [wavefront - 1][e / 4][lane]
     const int tid = threadIdx.x, lane = tid & 63;
@@ -632,14 +635,36 @@ __global__ __launch_bounds__(256) void k_conv_f4_small(const uint4* __restrict__
     auto ld16 = [](v4i& dst, const uint4* src) {
         asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(dst) : "v"(src) : "memory");
     };
+    v4i rsrc_x = {0, 0, 0, 0}, rsrc_w = {0, 0, 0, 0};
+    uint32_t wofs = 0u, xofs = 0u;
+    if constexpr (BUF) {
+        const uint64_t px = reinterpret_cast<uint64_t>(P4), pw = reinterpret_cast<uint64_t>(Wf);
+        rsrc_x = v4i{__builtin_amdgcn_readfirstlane((int)(uint32_t)px), __builtin_amdgcn_readfirstlane((int)((px >> 32) & 0xffffu)),
+                     __builtin_amdgcn_readfirstlane((int)p4_bytes), 0x00020000};
+        rsrc_w = v4i{__builtin_amdgcn_readfirstlane((int)(uint32_t)pw), __builtin_amdgcn_readfirstlane((int)((pw >> 32) & 0xffffu)),
+                     __builtin_amdgcn_readfirstlane((int)wf_bytes), 0x00020000};
+        wofs = ((uint32_t)min(kn0 / 32, rbmax) * (uint32_t)KB * 64u + (uint32_t)lane) * 16u;
+        xofs = ((pb + (uint32_t)(ih0 * cg.W + iw0)) * 2u + (uint32_t)h) * 16u;
+    }
+    auto ldbuf = [](v4i& dst, uint32_t voff, const v4i& rsrc, uint32_t soff) {
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(dst) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+    };
     auto load = [&](int w, Frag& f) {   // w is wave-uniform
         const int tap = (int)fastdiv((uint32_t)w, cg.dCP), ic = w - tap * cg.CP;
         const int kh = (int)fastdiv((uint32_t)tap, cg.dKW), kw = tap - kh * cg.KW;
-        ld16(f.w, wb + (size_t)w * 64);
         const int ih = ih0 + kh, iw = iw0 + kw;
-        f.in = (unsigned)ih < (unsigned)cg.H && (unsigned)iw < (unsigned)cg.W;
-        const size_t o = (size_t)(pb + (uint32_t)(ic * HWin + (f.in ? ih * cg.W + iw : 0))) * 2 + h;
-        ld16(f.x, P4 + o);
+        if constexpr (BUF) {
+            ldbuf(f.w, wofs, rsrc_w, (uint32_t)__builtin_amdgcn_readfirstlane(w) * 1024u);
+            const bool in = (unsigned)ih < (unsigned)cg.H && (unsigned)iw < (unsigned)cg.W;
+            const uint32_t tapoff = (uint32_t)__builtin_amdgcn_readfirstlane((ic * HWin + kh * cg.W + kw) * 32);
+            ldbuf(f.x, in ? xofs + tapoff : 0xffffff00u, rsrc_x, 0u);   // beyond p4_bytes: zeros
+            f.in = true;
+        } else {
+            ld16(f.w, wb + (size_t)w * 64);
+            f.in = (unsigned)ih < (unsigned)cg.H && (unsigned)iw < (unsigned)cg.W;
+            const size_t o = (size_t)(pb + (uint32_t)(ic * HWin + (f.in ? ih * cg.W + iw : 0))) * 2 + h;
+            ld16(f.x, P4 + o);
+        }
     };
     auto arrive = [](Frag& f, auto outstanding) {
         asm volatile("s_waitcnt vmcnt(%2)" : "+v"(f.w), "+v"(f.x) : "n"(decltype(outstanding)::value) : "memory");
@@ -647,7 +672,7 @@ __global__ __launch_bounds__(256) void k_conv_f4_small(const uint4* __restrict__
     auto compute = [&](const Frag& f) {
         v8i x, wv;
 #pragma unroll
-        for (int i = 0; i < 4; i++) x[i] = f.in ? f.x[i] : (int)fillv;
+        for (int i = 0; i < 4; i++) x[i] = (BUF || f.in) ? f.x[i] : (int)fillv;
 #pragma unroll
         for (int i = 4; i < 8; i++) x[i] = 0;
         wv = v8i{f.w[0], f.w[1], f.w[2], f.w[3], 0, 0, 0, 0};
@@ -825,21 +850,9 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
     const uint4* P4 = static_cast<const uint4*>(d_p4);
     const uint4* Wf = static_cast<const uint4*>(d_wf);
     const FastDiv dOHW = make_fastdiv((uint32_t)OHW);
-    // The kernel's hand-counted loads write registers behind the compiler's back; that is only
-    // sound while none of its registers live in scratch memory, which is checked once per variant.
-    auto launch = [&](auto variant) -> hipError_t {   // variant: a distinct type per kernel instance
-        constexpr auto kern = decltype(variant)::value;
-        static const hipError_t sound = []() {      // hence one check per instance
-            hipFuncAttributes attr;
-            hipError_t e = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(kern));
-            if (e == hipSuccess && attr.localSizeBytes != 0) e = hipErrorLaunchFailure;
-            return e;
-        }();
-        if (sound != hipSuccess) return sound;
-        hipLaunchKernelGGL(kern, grid, dim3(64 * wpb), 0, st, P4, Wf, d_y, (int)M, KN, OHW, KB, bias, alpha, dOHW, cg, qo);
-        return hipGetLastError();
-    };
-    // the 64 x 64 kernel takes two sizes more (its buffer-load variant announces them in its descriptors)
+    // The kernels' hand-counted loads write registers behind the compiler's back; that is only
+    // sound while none of their registers live in scratch memory, which is checked once per variant.
+    // operand sizes: the buffer-load variants announce them in their descriptors
     const int64_t p4_bytes = (int64_t)N * cg.CP * cg.H * cg.W * 32, wf_bytes = (int64_t)((KN + 31) / 32) * KB * 1024;
     static const bool no_buf = getenv("FTNN_CONV_NO_BUFFER_LOADS") != nullptr;   // tuning aid
     const bool buf = !no_buf && p4_bytes <= 0xf0000000LL && wf_bytes <= 0xf0000000LL;
@@ -868,7 +881,12 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
     auto by_split = [&](auto abin, auto form0, auto qmode) -> hipError_t {
         constexpr bool A = decltype(abin)::value, F = decltype(form0)::value;
         constexpr int Q = decltype(qmode)::value;
-        if (small) return launch(std::integral_constant<decltype(&k_conv_f4_small<A, F, Q>), &k_conv_f4_small<A, F, Q>>{});
+        if (small) {
+            if constexpr (!A) {
+                if (buf) return launch64(std::integral_constant<decltype(&k_conv_f4_small<A, F, Q, true>), &k_conv_f4_small<A, F, Q, true>>{});
+            }
+            return launch64(std::integral_constant<decltype(&k_conv_f4_small<A, F, Q, false>), &k_conv_f4_small<A, F, Q, false>>{});
+        }
         // three register sets: deeper prefetch measured no faster at any layer size
         if (split == 1) return by_buf(abin, form0, qmode, std::integral_constant<int, 1>{});
         if (split == 2) return by_buf(abin, form0, qmode, std::integral_constant<int, 2>{});
