@@ -342,16 +342,15 @@ struct ConvFrag {
 // All three are compile-time so that the per-element epilogue carries no selects for them.
 // The unsplit hand-over variants are the ones launched with several thousand wavefronts (stems,
 // first stages): they are asked to fit three wavefronts per SIMD, which they do without scratch.
-// BUF (ternary activations only): fragments arrive through buffer loads.  Their offsets are 32-bit, the weight
-// fragment of a word is addressed by a scalar offset alone, and an offset beyond the buffer returns zeros, which is
-// what a tap outside the image must contribute: no select on the loaded data, a third of the K loop's vector
-// instructions gone.  Needs both operands below 4 GiB (p4_bytes, wf_bytes: the sizes the descriptors announce).
+// BUF: fragments arrive through buffer loads.  Their offsets are 32-bit, the weight fragment of a word is addressed
+// by a scalar offset alone, and for ternary activations an offset beyond the buffer returns zeros, which is what a
+// tap outside the image must contribute: no select on the loaded data, a third of the K loop's vector instructions
+// gone (binary activations pad with +1 and keep the select).  Needs both operands below 4 GiB (p4_bytes, wf_bytes: the sizes the descriptors announce).
 template <bool ABIN, bool FORM0, int QMODE, int S, int NB, bool BUF>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && QMODE != 0) ? 3 : 1, 8))) void k_conv_f4(const uint4* __restrict__ P4, const uint4* __restrict__ Wf,
                                                  float* __restrict__ Y, int M, int KN, int OHW, int KB,
                                                  int bias, float alpha, FastDiv dOHW, ConvGeom cg, QuantOut qo,
                                                  uint32_t p4_bytes, uint32_t wf_bytes) {
-    static_assert(!(BUF && ABIN), "binary activations pad with +1, not with the zeros an out-of-range buffer load returns");
     // NB register sets of fragments: NB - 1 steps of loads in flight
     constexpr int WPB = 4;                // wavefronts per workgroup (single-wavefront workgroups for S = 1
                                           // measured slower: neighbours no longer share weight fragments in L1)
@@ -439,8 +438,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
             for (int b = 0; b < 2; b++) {
                 const int ih = ih0[b] + kh, iw = iw0[b] + kw;
                 const bool in = (unsigned)ih < (unsigned)cg.H && (unsigned)iw < (unsigned)cg.W;
-                ldbuf(f.x[b], in ? xofs[b] + tapoff : 0xffffff00u, rsrc_x, 0u);   // beyond p4_bytes: the load returns zeros
-                f.in[b] = true;
+                // ternary activations: an offset beyond p4_bytes returns the zeros that padding is; binary ones pad
+                // with +1, read record 0 instead and take the select in compute()
+                ldbuf(f.x[b], in ? xofs[b] + tapoff : (ABIN ? 0u : 0xffffff00u), rsrc_x, 0u);
+                f.in[b] = ABIN ? in : true;
             }
         } else {
 #pragma unroll
@@ -466,7 +467,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
 #pragma unroll
         for (int b = 0; b < 2; b++) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) x[b][i] = (BUF || f.in[b]) ? f.x[b][i] : (int)fillv;
+            for (int i = 0; i < 4; i++) x[b][i] = ((BUF && !ABIN) || f.in[b]) ? f.x[b][i] : (int)fillv;
 #pragma unroll
             for (int i = 4; i < 8; i++) x[b][i] = 0;
         }
@@ -602,7 +603,6 @@ __global__ __launch_bounds__(256) void k_conv_f4_small(const uint4* __restrict__
                                                        float* __restrict__ Y, int M, int KN, int OHW, int KB, int bias,
                                                        float alpha, FastDiv dOHW, ConvGeom cg, QuantOut qo,
                                                        uint32_t p4_bytes, uint32_t wf_bytes) {
-    static_assert(!(BUF && ABIN), "binary activations pad with +1");
     constexpr int S = 4, NB = 3;
     __shared__ float4 red[3 * 4 * 64];   // [wavefront - 1][e / 4][lane]
     const int tid = threadIdx.x, lane = tid & 63;
@@ -657,8 +657,8 @@ __global__ __launch_bounds__(256) void k_conv_f4_small(const uint4* __restrict__
             ldbuf(f.w, wofs, rsrc_w, (uint32_t)__builtin_amdgcn_readfirstlane(w) * 1024u);
             const bool in = (unsigned)ih < (unsigned)cg.H && (unsigned)iw < (unsigned)cg.W;
             const uint32_t tapoff = (uint32_t)__builtin_amdgcn_readfirstlane((ic * HWin + kh * cg.W + kw) * 32);
-            ldbuf(f.x, in ? xofs + tapoff : 0xffffff00u, rsrc_x, 0u);   // beyond p4_bytes: zeros
-            f.in = true;
+            ldbuf(f.x, in ? xofs + tapoff : (ABIN ? 0u : 0xffffff00u), rsrc_x, 0u);   // as in k_conv_f4
+            f.in = ABIN ? in : true;
         } else {
             ld16(f.w, wb + (size_t)w * 64);
             f.in = (unsigned)ih < (unsigned)cg.H && (unsigned)iw < (unsigned)cg.W;
@@ -672,7 +672,7 @@ __global__ __launch_bounds__(256) void k_conv_f4_small(const uint4* __restrict__
     auto compute = [&](const Frag& f) {
         v8i x, wv;
 #pragma unroll
-        for (int i = 0; i < 4; i++) x[i] = (BUF || f.in) ? f.x[i] : (int)fillv;
+        for (int i = 0; i < 4; i++) x[i] = ((BUF && !ABIN) || f.in) ? f.x[i] : (int)fillv;
 #pragma unroll
         for (int i = 4; i < 8; i++) x[i] = 0;
         wv = v8i{f.w[0], f.w[1], f.w[2], f.w[3], 0, 0, 0, 0};
@@ -872,9 +872,7 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
     auto by_buf = [&](auto abin, auto form0, auto qmode, auto sp) -> hipError_t {
         constexpr bool A = decltype(abin)::value, F = decltype(form0)::value;
         constexpr int Q = decltype(qmode)::value, SP = decltype(sp)::value;
-        if constexpr (!A) {
-            if (buf) return launch64(std::integral_constant<decltype(&k_conv_f4<A, F, Q, SP, 3, true>), &k_conv_f4<A, F, Q, SP, 3, true>>{});
-        }
+        if (buf) return launch64(std::integral_constant<decltype(&k_conv_f4<A, F, Q, SP, 3, true>), &k_conv_f4<A, F, Q, SP, 3, true>>{});
         return launch64(std::integral_constant<decltype(&k_conv_f4<A, F, Q, SP, 3, false>), &k_conv_f4<A, F, Q, SP, 3, false>>{});
     };
     // kernel variant: activation kind and PReLU form follow the type, then hand-over mode and split
@@ -882,9 +880,7 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
         constexpr bool A = decltype(abin)::value, F = decltype(form0)::value;
         constexpr int Q = decltype(qmode)::value;
         if (small) {
-            if constexpr (!A) {
-                if (buf) return launch64(std::integral_constant<decltype(&k_conv_f4_small<A, F, Q, true>), &k_conv_f4_small<A, F, Q, true>>{});
-            }
+            if (buf) return launch64(std::integral_constant<decltype(&k_conv_f4_small<A, F, Q, true>), &k_conv_f4_small<A, F, Q, true>>{});
             return launch64(std::integral_constant<decltype(&k_conv_f4_small<A, F, Q, false>), &k_conv_f4_small<A, F, Q, false>>{});
         }
         // three register sets: deeper prefetch measured no faster at any layer size
