@@ -644,11 +644,35 @@ hipError_t launch_pack_weights(bool ternary, const float* d_w, const float* d_th
     return hipGetLastError();
 }
 
+// bitpacking2 (src/utils.c:257-291) of rows of J = 256 * groups floats in {-1, 0, +1}.  A wavefront packs one group
+// of 256 values into its 4 sign and 4 zero words: lane l loads values l, 64 + l, 128 + l, 192 + l (four coalesced
+// loads in flight per lane), one ballot per load and plane is one word, and lanes 0..7 store the group's 64 bytes.
+// grid (rows, ceil(groups / 4)), block 256.
+__global__ __launch_bounds__(256) void k_pack_gemm_operand(const float* __restrict__ x, int J, int groups,
+                                                           unsigned long long* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int g = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const size_t r = blockIdx.x;
+    if (g >= groups) return;   // uniform per wavefront
+    const float* src = x + r * (size_t)J + (size_t)g * 256 + lane;
+    float v[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) v[c] = src[64 * c];
+    unsigned long long mine = 0;
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const unsigned long long s = __ballot(v[c] == -1.0f);
+        const unsigned long long z = ~__ballot(!(v[c] == 0.0f));
+        if (lane == c) mine = s;
+        if (lane == 4 + c) mine = z;
+    }
+    if (lane < 8) out[(r * (size_t)groups + (size_t)g) * 8 + lane] = mine;
+}
+
 hipError_t launch_pack_gemm_operand(const float* d_x, int I, int J, int64_t* d_out, hipStream_t st) {
-    const int words = J / 64;
-    dim3 grid(I, (words + 3) / 4);
-    hipLaunchKernelGGL((k_quantize_ballot<2, true>), grid, dim3(256), 0, st, d_x,
-                       (const float*)nullptr, J, words,
+    const int groups = J / 256;   // the caller has checked J % 256 == 0
+    dim3 grid(I, (groups + 3) / 4);
+    hipLaunchKernelGGL(k_pack_gemm_operand, grid, dim3(256), 0, st, d_x, J, groups,
                        reinterpret_cast<unsigned long long*>(d_out));
     return hipGetLastError();
 }

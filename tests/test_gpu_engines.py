@@ -53,6 +53,17 @@ def test_engines_on_gemm_operands(hip, oracle, mnp):
         assert got.tobytes() == want.tobytes(), "engine %d" % eng
 
 
+@pytest.mark.parametrize("rows,cols", [(1, 256), (3, 1280), (70, 768), (257, 4096), (5, 256 * 9)])
+def test_gemm_operand_packer_matches_bitpacking2(hip, oracle, rows, cols):
+    """ftnn_pack_gemm_operand against the oracle's bitpacking2 (src/utils.c:257-291), word for word: one group of 256
+    values, group counts that leave the last workgroup partly idle, several rows"""
+    from fastertnn_amd import synth
+    x = synth.ternary(rows * 7 + cols, (rows, cols))
+    want = oracle.pack_gemm_operand(x)
+    got = hip.pack_gemm_operand(_dev(x)).cpu().numpy()
+    assert got.tobytes() == np.ascontiguousarray(want).tobytes()
+
+
 @pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
 @pytest.mark.parametrize("mnk", [(1, 64, 4), (5, 65, 8), (70, 100, 12), (200, 257, 36), (1000, 64, 4),
                                  (129, 1000, 8), (64, 63, 4), (300, 2048, 20)])
