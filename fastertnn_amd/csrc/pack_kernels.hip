@@ -211,47 +211,59 @@ __global__ __launch_bounds__(256) void k_im2row(const unsigned long long* __rest
 }
 
 // ------------------------------------------------------------- weight packers
-// one work-item per output word; w is fp32 (KN, C, KH, KW)
+// w is fp32 (KN, C, KH, KW).  A wavefront packs the words of one (kernel n, channel word ic): lane = channel within
+// the word, one ballot per tap and plane.  The taps of a channel are neighbours in memory, so a wavefront meets the
+// same cache lines again from tap to tap, and four taps' loads leave before the first is used.  The wavefront of
+// ic = 0 also writes the padding words that round a row up to a multiple of 4.
+// grid ceil(KN * CP / 4), block 256.
 template <bool TERN>
 __global__ __launch_bounds__(256) void k_pack_weights(const float* __restrict__ w,
                                                       const float* __restrict__ thr, int C,
                                                       int taps, int CP, int K, int Kw,
-                                                      int64_t total,
+                                                      int64_t pairs,
                                                       unsigned long long* __restrict__ out) {
-    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (e >= total) return;
-    const int64_t n = e / Kw;
-    const int idx = (int)(e - n * Kw);
-    unsigned long long s = 0ull, z = TERN ? ~0ull : 0ull;
-    if (idx < K) {
-        const int ic = idx % CP, tap = idx / CP;
-        const float t = thr[n];
-        z = 0ull;
-        for (int bit = 0; bit < 64; bit++) {
-            const int c = ic * 64 + bit;
+    const int lane = threadIdx.x & 63;
+    const int64_t e = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);   // (n, ic), uniform per wavefront
+    if (e >= pairs) return;
+    const int64_t n = e / CP;
+    const int ic = (int)(e - n * CP);
+    const int c = ic * 64 + lane;
+    const bool real = c < C;
+    const float t = thr[n];
+    const float* src = w + ((size_t)n * C + (real ? c : 0)) * taps;
+    unsigned long long* row = out + (size_t)n * (TERN ? 2 : 1) * Kw;
+    for (int tap0 = 0; tap0 < taps; tap0 += 4) {
+        float v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] = (real && tap0 + k < taps) ? src[tap0 + k] : 0.0f;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            if (tap0 + k >= taps) break;   // uniform
+            const int idx = (tap0 + k) * CP + ic;
             if (TERN) {
-                // channels past C read as 0.0 and take the same compares, positive side
-                // first (src/utils.c:498-509)
-                const float v = c < C ? w[((size_t)n * C + c) * taps + tap] : 0.0f;
-                if (v > t) {
-                } else if (v < -t) {
-                    s |= 1ull << bit;
-                } else {
-                    z |= 1ull << bit;
+                // channels past C read as 0.0 and take the same compares, positive side first (src/utils.c:498-509)
+                const bool pos = v[k] > t;
+                const bool neg = !pos && v[k] < -t;
+                const unsigned long long s = __ballot(neg), z = __ballot(!pos && !neg);
+                if (lane == 0) {
+                    row[p2_pos(idx, 0)] = s;
+                    row[p2_pos(idx, 1)] = z;
                 }
-            } else if (c < C) {
-                // src/utils.c:654-660
-                const float v = w[((size_t)n * C + c) * taps + tap];
-                if (v < t) s |= 1ull << bit;
+            } else {
+                const unsigned long long s = __ballot(real && v[k] < t);   // src/utils.c:654-660
+                if (lane == 0) row[idx] = s;
             }
         }
     }
-    if (TERN) {
-        unsigned long long* row = out + (size_t)n * 2 * Kw;
-        row[p2_pos(idx, 0)] = s;
-        row[p2_pos(idx, 1)] = z;
-    } else {
-        out[(size_t)n * Kw + idx] = s;
+    // padding words: (sign 0, zero all ones) for ternary rows (src/utils.c:483-490), 0 for binary ones (:643-647)
+    if (ic == 0 && lane < Kw - K) {
+        const int idx = K + lane;
+        if (TERN) {
+            row[p2_pos(idx, 0)] = 0ull;
+            row[p2_pos(idx, 1)] = ~0ull;
+        } else {
+            row[idx] = 0ull;
+        }
     }
 }
 
@@ -632,15 +644,16 @@ hipError_t launch_quantize_im2row(bool ternary, const float* d_x, const float* d
 hipError_t launch_pack_weights(bool ternary, const float* d_w, const float* d_thr, int KN, int C,
                                int KH, int KW, int64_t* d_out, hipStream_t st) {
     const int CP = cpack_of(C), K = CP * KH * KW, Kw = round4(K);
-    const int64_t total = (int64_t)KN * Kw;
-    const unsigned blocks = (unsigned)((total + 255) / 256);
+    const int64_t pairs = (int64_t)KN * CP;   // (kernel, channel word)
+    if ((pairs + 3) / 4 > 0x7fffffffLL) return hipErrorInvalidValue;
+    const unsigned blocks = (unsigned)((pairs + 3) / 4);
     unsigned long long* out = reinterpret_cast<unsigned long long*>(d_out);
     if (ternary)
         hipLaunchKernelGGL((k_pack_weights<true>), dim3(blocks), dim3(256), 0, st, d_w, d_thr, C,
-                           KH * KW, CP, K, Kw, total, out);
+                           KH * KW, CP, K, Kw, pairs, out);
     else
         hipLaunchKernelGGL((k_pack_weights<false>), dim3(blocks), dim3(256), 0, st, d_w, d_thr, C,
-                           KH * KW, CP, K, Kw, total, out);
+                           KH * KW, CP, K, Kw, pairs, out);
     return hipGetLastError();
 }
 

@@ -53,6 +53,24 @@ def test_engines_on_gemm_operands(hip, oracle, mnp):
         assert got.tobytes() == want.tobytes(), "engine %d" % eng
 
 
+@pytest.mark.parametrize("ternary", [True, False], ids=["ternary", "binary"])
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1), (5, 3, 7, 7), (64, 64, 3, 3), (33, 65, 1, 1), (7, 130, 5, 2),
+                                   (130, 127, 3, 3), (3, 200, 1, 7), (2, 64, 2, 3)])
+def test_weight_packer_matches_the_oracle(hip, oracle, ternary, shape):
+    """ftnn_pack_weights against the oracle's ternarize_opt / binarize_opt restatement (src/utils.c:468-521, 634-675),
+    word for word: channel tails, tap counts that are no multiple of the four loaded together, padding words, and
+    thresholds of either sign (a negative ternary threshold turns the channels past C into +1, as in the reference)"""
+    from fastertnn_amd import synth
+    kn, c, kh, kw = shape
+    w = synth.normal(kn * 31 + c, (kn, c, kh, kw))
+    for thr_value in (0.5, 0.0, -0.25):
+        thr = np.full(kn, thr_value, np.float32)
+        thr[::2] *= 0.5
+        want = oracle.pack_weights(w, thr, ternary)
+        got = hip.pack_weights(_dev(w), _dev(thr), ternary).cpu().numpy()
+        assert got.tobytes() == np.ascontiguousarray(want).tobytes(), thr_value
+
+
 @pytest.mark.parametrize("rows,cols", [(1, 256), (3, 1280), (70, 768), (257, 4096), (5, 256 * 9)])
 def test_gemm_operand_packer_matches_bitpacking2(hip, oracle, rows, cols):
     """ftnn_pack_gemm_operand against the oracle's bitpacking2 (src/utils.c:257-291), word for word: one group of 256
