@@ -16,6 +16,8 @@
 
 #include <type_traits>
 
+#include <stdlib.h>
+
 #include "ftnn_internal.h"
 
 namespace ftnn {
@@ -25,7 +27,7 @@ namespace {
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int kTile = 16;   // output pixels per workgroup: kTile x kTile, 4 rows of 16 per wavefront
+constexpr int kTile = 16;   // output pixels per workgroup: kTile wide, 4 rows per wavefront (16 rows with four wavefronts)
 
 struct StemGeom {
     int C, H, W, OH, OW, KW, taps, Kd;
@@ -62,7 +64,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
     const int h = lane >> 5, lr = lane & 31;
     const int n = blockIdx.z, kn0 = blockIdx.y * 64;
     const int ty = (int)fastdiv(blockIdx.x, g.dTX), tx = (int)blockIdx.x - ty * g.tiles_x;
-    const int oh0 = ty * kTile, ow0 = tx * kTile;
+    const int NT = blockDim.x;   // 64 per wavefront: a tile is 4 rows of kTile pixels per wavefront
+    const int oh0 = ty * (int)(blockDim.x >> 4), ow0 = tx * kTile;
     const int HW = g.H * g.W;
 
     // ---- the patch: quantise on the way into LDS ----
@@ -78,21 +81,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
         uint4 wreg[kWR];
 #pragma unroll
         for (int k = 0; k < kWR; k++) {
-            const int i = min(tid + 256 * k, nwf - 1);
+            const int i = min(tid + NT * k, nwf - 1);
             const int d = i >> 7, a = (i >> 6) & 1, l = i & 63;
             wreg[k] = Wf[((size_t)min(kn0 / 32 + a, rbm) * KB + d) * 64 + l];
         }
         // kCH patch pixels per thread and round, all their loads issued before the first is used: the fill is a
         // chain of memory latencies otherwise (one round covers the 37 x 37 patch of a stride-2 7x7 layer)
         constexpr int kCH = 6;
-        for (int base = 0; base < PP; base += 256 * kCH) {
+        for (int base = 0; base < PP; base += NT * kCH) {
             float v[kCH][C];
             bool in[kCH];
 #pragma unroll
             for (int k = 0; k < kCH; k++) {
                 in[k] = false;
-                if (base + 256 * k < PP) {   // wave-uniform up to the last 256 pixels
-                    const int idx = min(base + 256 * k + tid, PP - 1);
+                if (base + NT * k < PP) {   // wave-uniform up to the last 256 pixels
+                    const int idx = min(base + NT * k + tid, PP - 1);
                     const int py = (int)fastdiv((uint32_t)idx, g.dPW), px = idx - py * g.PW;
                     const int ih = ihb + py, iw = iwb + px;
                     in[k] = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
@@ -103,7 +106,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
             }
 #pragma unroll
             for (int k = 0; k < kCH; k++) {
-                const int idx = base + 256 * k + tid;
+                const int idx = base + NT * k + tid;
                 if (idx < PP) {
                     uint32_t dw = 0u;
 #pragma unroll
@@ -120,12 +123,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
         }
 #pragma unroll
         for (int k = 0; k < kWR; k++)
-            if (tid + 256 * k < nwf) wl[tid + 256 * k] = wreg[k];
-        for (int i = tid + 256 * kWR; i < nwf; i += 256) {   // more than 4 words: the rest, one by one
+            if (tid + NT * k < nwf) wl[tid + NT * k] = wreg[k];
+        for (int i = tid + NT * kWR; i < nwf; i += NT) {   // more than 4 words: the rest, one by one
             const int d = i >> 7, a = (i >> 6) & 1, l = i & 63;
             wl[i] = Wf[((size_t)min(kn0 / 32 + a, rbm) * KB + d) * 64 + l];
         }
-        for (int idx = tid; idx < g.Kd * TT; idx += 256) {
+        for (int idx = tid; idx < g.Kd * TT; idx += NT) {
             const int d = idx / TT, j = idx - d * TT;
             const int tap = d * T + j;
             uint32_t off = (uint32_t)PP;   // a tap that does not exist reads the padding region
@@ -243,30 +246,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
 
 // LDS the kernel needs for this layer, or 0 where the fused first-layer kernel does not apply (more than 8
 // channels, or an input patch beyond the 64 KiB a workgroup gets without opting in)
-int64_t stem_f4_lds_bytes(int C, int KH, int KW, int H_stride, int W_stride) {
+static int64_t stem_lds_bytes_for(int C, int KH, int KW, int H_stride, int W_stride, int waves) {
     if (C < 1 || C > 8) return 0;
     const int T = 64 / C, J1 = 32 / C, NI0 = (32 + C - 1) / C, NI = NI0 > T - J1 ? NI0 : T - J1;
-    const int64_t PH = (int64_t)(kTile - 1) * H_stride + KH, PW = (int64_t)(kTile - 1) * W_stride + KW;
+    const int64_t PH = (int64_t)(4 * waves - 1) * H_stride + KH, PW = (int64_t)(kTile - 1) * W_stride + KW;
     const int64_t Kd = ((int64_t)KH * KW + T - 1) / T;
     // patch and padding, tap table (rounded up to 16 bytes), weight fragments of one kernel tile
     const int64_t bytes = ((2 * PH * PW + Kd * (J1 + NI) + 3) / 4 * 4) * 4 + Kd * 2 * 1024;
     return bytes <= 64 * 1024 ? bytes : 0;
 }
 
+// the layer runs in the fused kernel if its patch fits with the smaller tile (two wavefronts, 8 rows)
+int64_t stem_f4_lds_bytes(int C, int KH, int KW, int H_stride, int W_stride) {
+    return stem_lds_bytes_for(C, KH, KW, H_stride, W_stride, 2);
+}
+
 hipError_t launch_stem_f4(int type, const float* d_x, const float* d_thr, const void* d_wf, int N, int C, int H,
                           int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride, int W_stride,
                           float alpha, float* d_y, hipStream_t st, const QuantOut& qo) {
-    const int64_t lds_bytes = stem_f4_lds_bytes(C, KH, KW, H_stride, W_stride);
-    if (lds_bytes == 0) return hipErrorInvalidValue;
     const int OH = out_dim(H, H_pad, KH, H_stride), OW = out_dim(W, W_pad, KW, W_stride);
+    // wavefronts per workgroup = tile height / 4 (tuning aid: FTNN_STEM_WAVES)
+    static const int forced = getenv("FTNN_STEM_WAVES") ? atoi(getenv("FTNN_STEM_WAVES")) : 0;
+    int waves = 4;
+    if (forced == 2 || forced == 4) waves = forced;
+    if (stem_lds_bytes_for(C, KH, KW, H_stride, W_stride, waves) == 0) waves = 2;
+    const int64_t lds_bytes = stem_lds_bytes_for(C, KH, KW, H_stride, W_stride, waves);
+    if (lds_bytes == 0) return hipErrorInvalidValue;
+    const int tile_h = 4 * waves;
     const int T = 64 / C, taps = KH * KW, Kd = (taps + T - 1) / T;
     StemGeom g;
     g.C = C; g.H = H; g.W = W; g.OH = OH; g.OW = OW; g.KW = KW; g.taps = taps; g.Kd = Kd;
     g.H_pad = H_pad; g.W_pad = W_pad; g.H_stride = H_stride; g.W_stride = W_stride;
-    g.PH = (kTile - 1) * H_stride + KH;
+    g.PH = (tile_h - 1) * H_stride + KH;
     g.PW = (kTile - 1) * W_stride + KW;
     g.tiles_x = (OW + kTile - 1) / kTile;
-    const int tiles_y = (OH + kTile - 1) / kTile;
+    const int tiles_y = (OH + tile_h - 1) / tile_h;
     g.dPW = make_fastdiv((uint32_t)g.PW);
     g.dKW = make_fastdiv((uint32_t)KW);
     g.dTX = make_fastdiv((uint32_t)g.tiles_x);
@@ -283,7 +297,7 @@ hipError_t launch_stem_f4(int type, const float* d_x, const float* d_thr, const 
         constexpr int Q = decltype(qmode)::value;
 #define FTNN_STEM(C_)                                                                                         \
     case C_:                                                                                                  \
-        hipLaunchKernelGGL((k_stem_f4<A, F, Q, C_>), grid, dim3(256), (size_t)lds_bytes, st, d_x, d_thr, Wf, d_y, KN, \
+        hipLaunchKernelGGL((k_stem_f4<A, F, Q, C_>), grid, dim3(64 * waves), (size_t)lds_bytes, st, d_x, d_thr, Wf, d_y, KN, \
                            KB, bias, alpha, g, qo);                                                           \
         break;
         switch (C) {
