@@ -2,7 +2,7 @@
 (fastertnn_amd/csrc/stem_kernels.hip).  Every channel count (each has its own word layout: T = 64 / C taps per
 word, the upper half of a word starting mid-tap when C does not divide 32), every type, windows whose taps do and
 do not fill their last word, tiles that overhang the image, kernel counts that are no multiple of 32; fp32 results
-and all hand-over forms; and the two-kernel form that takes over when the input patch of a tile exceeds the LDS."""
+and all hand-over forms; and the smaller tile and the two-kernel form that take over when the input patch of a tile exceeds the LDS."""
 import numpy as np
 import pytest
 
@@ -70,15 +70,18 @@ def test_first_layer_hand_over(hip, oracle, c):
             assert got.tobytes() == want.tobytes()
 
 
-def test_patch_larger_than_the_lds_takes_the_two_kernel_form(hip, oracle):
-    """stride 8 with a 3x3 window: the input patch of a 16 x 16 output tile is 123 x 123 pixels, beyond the LDS of a
-    workgroup, so the layer runs as nibble quantiser + per-pixel rows + 1x1 fp4 layer; same bits"""
+@pytest.mark.parametrize("stride,what", [(8, "16 x 8 tiles"), (12, "two-kernel form")])
+def test_patches_larger_than_the_lds(hip, oracle, stride, what):
+    """a 3x3 window at stride 8: the input patch of a 16 x 16 output tile is 123 x 123 pixels, beyond the LDS of a
+    workgroup, and the layer runs on tiles of 16 x 8 pixels (two wavefronts); at stride 12 that patch is too large as
+    well and the layer runs as nibble quantiser + per-pixel rows + 1x1 fp4 layer; same bits either way"""
     import torch
     for typ in ALL_TYPES:
-        shape = (3, 75, 91, 64, 3, 3, 1, 8)
+        shape = (3, 75, 91, 64, 3, 3, 1, stride)
+        print("case", what, TYPE_NAMES[typ], shape, flush=True)
         L = make_layer(typ, shape, 2, seed=77 + typ)
         qw = oracle.pack_weights(L["w"], L["wthr"], weight_is_ternary(typ))
-        want = oracle.conv(typ, L["x"], L["thr"], qw, 64, 3, 3, 1, 8, 0.5)
+        want = oracle.conv(typ, L["x"], L["thr"], qw, 64, 3, 3, 1, stride, 0.5)
         got = hip.conv(typ, torch.from_numpy(L["x"]).cuda(), torch.from_numpy(L["thr"]).cuda(),
-                       torch.from_numpy(qw).cuda(), 64, 3, 3, 1, 8, 0.5, engine=hip.ENGINE_MFMA_F4)
+                       torch.from_numpy(qw).cuda(), 64, 3, 3, 1, stride, 0.5, engine=hip.ENGINE_MFMA_F4)
         assert got.cpu().numpy().tobytes() == np.ascontiguousarray(want).tobytes()
