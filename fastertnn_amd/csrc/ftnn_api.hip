@@ -862,7 +862,7 @@ void tnns_conv(testcase_t* t) {
     if (check_conv_shape(N, C, H, W, t->paddingH, t->paddingW, KH, KW, t->strideH, t->strideW, &OH,
                          &OW) != FTNN_OK || KN <= 0)
         die("tnns_conv");
-    const int act_tern = (type == kTNN || type == kTBN), w_tern = (type == kTNN || type == kBTN);
+    const int w_tern = (type == kTNN || type == kBTN);
     const size_t rows = (size_t)N * OH * OW;
     float* d_x = (float*)upload(SLOT_X, t->input, (size_t)N * C * H * W * sizeof(float));
     float* d_thr = (float*)upload(SLOT_THR, t->input_thresholds, (size_t)N * sizeof(float));
