@@ -276,14 +276,6 @@ def conv_latency(torch, lib, typ, shape, batch, seed, reps=20):
     return out
 
 
-RESNET18_LIKE = [  # (C, IH, IW, KN, KW, KH, pad, stride): stem, four stages with stride-2 transitions, FC as 1x1
-    (3, 224, 224, 64, 7, 7, 3, 2), (64, 112, 112, 64, 3, 3, 1, 2),
-    (64, 56, 56, 64, 3, 3, 1, 1), (64, 56, 56, 64, 3, 3, 1, 1), (64, 56, 56, 64, 3, 3, 1, 1), (64, 56, 56, 64, 3, 3, 1, 1),
-    (64, 56, 56, 128, 3, 3, 1, 2), (128, 28, 28, 128, 3, 3, 1, 1), (128, 28, 28, 128, 3, 3, 1, 1), (128, 28, 28, 128, 3, 3, 1, 1),
-    (128, 28, 28, 256, 3, 3, 1, 2), (256, 14, 14, 256, 3, 3, 1, 1), (256, 14, 14, 256, 3, 3, 1, 1), (256, 14, 14, 256, 3, 3, 1, 1),
-    (256, 14, 14, 512, 3, 3, 1, 2), (512, 7, 7, 512, 3, 3, 1, 1), (512, 7, 7, 512, 3, 3, 1, 1), (512, 7, 7, 512, 3, 3, 1, 1),
-    (512, 7, 7, 1000, 1, 1, 0, 1),
-]
 
 
 def e2e_latency(torch, lib, batch, reps=50, cpu=True, typ=None):
@@ -291,6 +283,7 @@ def e2e_latency(torch, lib, batch, reps=50, cpu=True, typ=None):
     (cpu=True) the same chain through the reference's tnns_conv on one host core"""
     import numpy as np
     from fastertnn_amd import TNN, act_is_ternary, weight_is_ternary
+    from fastertnn_amd.shapes import RESNET18_LIKE
     typ = TNN if typ is None else typ
     at, wt = act_is_ternary(typ), weight_is_ternary(typ)
     g = torch.Generator(device="cuda")
@@ -385,13 +378,13 @@ def reference_gemm_sweep(torch, lib, reps=10):
 
 def reference_single_layers(torch, lib, batch=8, reps=10):
     """the 17 layers of the reference's `layer` mode (include/timing/shapes_layers.h, kept as data in
-    tests/golden/reference_shape_tables.json), TNN, batch 8 (src/timing_layers.c:46): device-resident call with
+    fastertnn_amd/data/reference_shape_tables.txt), TNN, batch 8 (src/timing_layers.c:46): device-resident call with
     prepared weights against the reference's tnns_conv on one host core"""
     import numpy as np
     from fastertnn_amd import TNN
     from oracle import ftnn_oracle as O
-    tables = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "golden",
-                                         "reference_shape_tables.json")))
+    from fastertnn_amd import shapes
+    tables = shapes.reference_tables()
     out = {}
     g = torch.Generator(device="cuda")
     g.manual_seed(9)
@@ -429,15 +422,15 @@ def reference_single_layers(torch, lib, batch=8, reps=10):
 
 def reference_networks(torch, lib, batch=8, reps=5):
     """the seven networks of the reference's e2e mode (include/timing/shapes_e2e.h, kept as data in
-    tests/golden/reference_shape_tables.json), at the reference's batch of 8 (src/timing_layers.c:46): device-resident
+    fastertnn_amd/data/reference_shape_tables.txt), at the reference's batch of 8 (src/timing_layers.c:46): device-resident
     layer chain against the same tnns_conv chain on one host core.  Three tables leave out their pooling layers; there
     the reference's driver hands the previous output buffer on under the next row's shape
     (src/timing_layers.c:187-200), and so do the chain (FTNN_NET_REREAD_PREFIX) and the CPU side here."""
     import numpy as np
     from fastertnn_amd import TNN
     from oracle import ftnn_oracle as O
-    tables = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "golden",
-                                         "reference_shape_tables.json")))
+    from fastertnn_amd import shapes
+    tables = shapes.reference_tables()
     out = {}
     g = torch.Generator(device="cuda")
     g.manual_seed(8)

@@ -37,6 +37,49 @@ def test_large_tnn_gemm_properties(hip, oracle):
     assert y05[rows].cpu().numpy().tobytes() == want.tobytes()
 
 
+def test_large_tnn_gemm_on_every_engine(hip, oracle):
+    """M = N = 8192, K = 32768 on independent uniform ternary operands, PReLU 0.5: the engine AUTO resolves to is
+    the fp4 matrix-core one (512 K words through its LDS ring), and AUTO, fp4 and int8 give the vector-ALU
+    engine's bits on every element; rows from different tiles and wavefronts are bit-exact against the oracle
+    (src/tnns/mm_p2_final_tnn_avx2.c:384-387)"""
+    import torch
+    m = n = 8192
+    k = 32768
+    kw = k // 64
+    ops = []
+    for seed in (5, 6):
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        packed = torch.empty(m * k // 32, dtype=torch.int64, device="cuda")
+        for r0 in range(0, m, 2048):   # 256 MiB of fp32 at a time
+            x = torch.randint(-1, 2, (2048, k), generator=g, device="cuda", dtype=torch.int8).float()
+            packed[r0 * k // 32:(r0 + 2048) * k // 32] = hip.pack_gemm_operand(x)
+        ops.append(packed)
+    a, b = ops
+    assert hip.select_engine(TNN, m, 1, 1, n, kw) == hip.ENGINE_MFMA_F4
+    need = max(hip.mm_scratch_bytes(e, TNN, m, 1, 1, n, kw) for e in (hip.ENGINE_MFMA_I8, hip.ENGINE_MFMA_F4))
+    assert hip.mm_scratch_bytes(hip.ENGINE_AUTO, TNN, m, 1, 1, n, kw) == hip.mm_scratch_bytes(hip.ENGINE_MFMA_F4, TNN, m, 1, 1, n, kw)
+    scratch = torch.empty(need, dtype=torch.uint8, device="cuda")
+    ref = hip.mm_engine(hip.ENGINE_VALU, TNN, a, b, m, 1, 1, n, kw, 0.5)
+    rows = [0, 31, 32, 127, 128, 255, 256, 4097, 6000, 8191]
+    ah = a.view(m, 2 * kw)[rows].cpu().numpy()
+    want = oracle.mm(TNN, np.ascontiguousarray(ah).reshape(-1), b.cpu().numpy(), len(rows), 1, 1, n, kw, 0.5)
+    assert ref.view(m, n)[rows].cpu().numpy().tobytes() == np.ascontiguousarray(want).tobytes()
+    for eng in (hip.ENGINE_AUTO, hip.ENGINE_MFMA_F4, hip.ENGINE_MFMA_I8):
+        print("engine", eng, flush=True)
+        y = torch.full((m, n, 1, 1), float("nan"), dtype=torch.float32, device="cuda")
+        scratch.fill_(0x5a)
+        hip.mm_engine(eng, TNN, a, b, m, 1, 1, n, kw, 0.5, out=y, scratch=scratch)
+        assert torch.equal(y.view(torch.int32), ref.view(torch.int32)), "engine %d" % eng
+        del y
+    # a caller that keeps the weights expanded (ftnn_expand_rows once, ftnn_mm_expanded per call) gets the same bits
+    for eng in (hip.ENGINE_MFMA_F4, hip.ENGINE_MFMA_I8):
+        a_exp, b_exp = hip.expand_rows(eng, a, m, kw, True), hip.expand_rows(eng, b, n, kw, True)
+        y = hip.mm_expanded(eng, TNN, a_exp, b_exp, m, 1, 1, n, kw, 0.5)
+        assert torch.equal(y.view(torch.int32), ref.view(torch.int32)), "expanded, engine %d" % eng
+        del a_exp, b_exp, y
+
+
 @pytest.mark.parametrize("typ", [TNN, TBN, BTN, BNN], ids=lambda t: TYPE_NAMES[t])
 def test_resnet_stage_layers_batch32(hip, oracle, typ):
     """the 3x3 stage layers of the batch-32 stack (C=64@56x56 ... C=512@7x7): the fused layer

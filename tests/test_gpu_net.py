@@ -195,3 +195,44 @@ def test_random_chains_match_the_oracle(hip, oracle):
         net.close()
         assert got.tobytes() == np.ascontiguousarray(want).tobytes()
         done += 1
+
+
+def test_resnet18_like_stack_at_batch_32(hip, oracle):
+    """The end-to-end configuration at its stated size: batch 32, 3 x 224 x 224 fp32 N(0,1) input, the 19 layers of
+    the ResNet-18-like TNN stack (thresholds 0.5, uniform ternary weights, PReLU 0.5), chained on the device with the
+    quantised hand-over between layers.  Eager launches and HIP-graph replays give the same bits; sampled images are
+    bit-exact against the oracle's layer-by-layer chain (images of a batch never meet, so a chain over a sub-batch
+    is exact), and the whole batch against the reference's own tnns_conv chain where its compiled form is present
+    (src/timing_layers.c:182-207)."""
+    import torch
+    from fastertnn_amd.shapes import RESNET18_LIKE
+    from oracle.ftnn_oracle import Reference, aligned_copy
+    batch = 32
+    stack = [(TNN, row) for row in RESNET18_LIKE]
+    net, host = build(hip, oracle, batch, stack)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(6)
+    xd = torch.randn((batch, 3, 224, 224), generator=g, device="cuda")
+    got = net.run(xd)
+    torch.cuda.synchronize()
+    assert got.shape == (batch, 1000, 7, 7)   # the fully connected layer is the 1x1 layer of the reference's table, on 7 x 7 pixels
+    s = torch.cuda.Stream()
+    out = torch.empty_like(got)
+    with torch.cuda.stream(s):
+        for rep in range(3):
+            out.fill_(-1.0)
+            net.run(xd, out=out, graph=True)
+            s.synchronize()
+            assert torch.equal(out.view(torch.int32), got.view(torch.int32)), "replay %d" % rep
+    net.close()
+    imgs = [0, 13, 31]
+    print("oracle chain on images", imgs, flush=True)
+    want = oracle_chain(oracle, host, xd[imgs].cpu().numpy())
+    assert got[imgs].cpu().numpy().tobytes() == np.ascontiguousarray(want).tobytes()
+    if Reference.available():
+        print("reference chain on the whole batch", flush=True)
+        ref = Reference()
+        xh = xd.cpu().numpy()
+        for typ, (c, ih, iw, kn, kw, kh, pad, stride), qw, thr in host:
+            xh = ref.conv(typ, xh, np.full(batch, thr, np.float32), aligned_copy(qw), kn, kh, kw, pad, stride, 0.5)
+        assert got.cpu().numpy().tobytes() == np.ascontiguousarray(xh).tobytes()

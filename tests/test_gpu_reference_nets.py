@@ -1,21 +1,17 @@
-"""The networks of the reference's e2e mode (include/timing/shapes_e2e.h via tests/golden/reference_shape_tables.json)
+"""The networks of the reference's e2e mode (include/timing/shapes_e2e.h, kept as data in fastertnn_amd/data/reference_shape_tables.txt)
 as device-resident layer chains (ftnn_net_*), against the same chain of tnns_conv calls on the CPU
 (src/timing_layers.c:182-207): bit-identical final activations.  Four of the seven tables chain shape to shape
 (ResNet-18, Darknet-19, Darknet-53, ResNet-152); the other three leave out their pooling layers, the reference's
 driver re-reads a prefix of the previous buffer there (src/timing_layers.c:187-200); a layer chain rejects them unless
 it is created with FTNN_NET_REREAD_PREFIX, and then does the same."""
-import json
-import os
-
 import numpy as np
 import pytest
 
-from fastertnn_amd import synth, TNN, TBN, BTN, BNN, TYPE_NAMES, act_is_ternary, weight_is_ternary
+from fastertnn_amd import shapes, synth, TNN, TBN, BTN, BNN, TYPE_NAMES, act_is_ternary, weight_is_ternary
 
 pytestmark = pytest.mark.gpu
 
-TABLES = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
-                                     "reference_shape_tables.json")))
+TABLES = shapes.reference_tables()
 NETS = {n["name"]: [tuple(r) for r in n["layers"]] for n in TABLES["e2e"]}
 CHAINABLE = ["resnet18", "darknet19", "darknet53", "resnet152"]
 
