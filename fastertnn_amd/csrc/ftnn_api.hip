@@ -472,6 +472,44 @@ int conv_valu(int type, const float* d_x, const float* d_thr, const int64_t* d_q
     return e == hipSuccess ? FTNN_OK : hip_fail(e, "implicit-im2row mm launch");
 }
 
+// ---- the scratch memory of ftnn_conv_static ----
+// Device memory that exists from the moment the code object is loaded until the process ends, one copy per GPU,
+// so that a caller who may not allocate (a stream under graph capture, a serving loop, a harness that forbids
+// hipMalloc) still has somewhere to put a layer's quantised input and weight fragments.  `scratch` is the
+// host-side handle of that array, not a device address: the address of each GPU's copy comes from
+// hipGetSymbolAddress, once per device, and is what every launch below is given.
+constexpr int64_t kStaticScratchBytes = FTNN_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void* g_static_scratch[kMaxDevices] = {};
+static std::mutex g_static_scratch_mutex;
+
+// address of the current device's copy of `scratch`; nullptr (and the error text set) on failure
+static void* static_scratch_of_current_device() {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        hip_fail(e, "hipGetDevice");
+        return nullptr;
+    }
+    if (dev < 0 || dev >= kMaxDevices) {
+        fail(FTNN_EINVAL, "device ordinal %d beyond the %d this library keeps scratch for", dev, kMaxDevices);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+    if (!g_static_scratch[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            hip_fail(e, "hipGetSymbolAddress(scratch)");
+            return nullptr;
+        }
+        g_static_scratch[dev] = ptr;
+    }
+    return g_static_scratch[dev];
+}
+
 }  // namespace ftnn
 
 using namespace ftnn;
@@ -798,6 +836,24 @@ int ftnn_conv(int type, const float* d_x, const float* d_thr, const int64_t* d_q
               float prelu_alpha, void* d_scratch, float* d_y, void* stream) {
     return ftnn_conv_engine(FTNN_ENGINE_AUTO, type, d_x, d_thr, d_qw, N, C, H, W, KN, KH, KW, H_pad, W_pad,
                             H_stride, W_stride, prelu_alpha, d_scratch, d_y, stream);
+}
+
+int ftnn_conv_static(int type, const float* d_x, const float* d_thr, const int64_t* d_qw, int N, int C, int H, int W,
+                     int KN, int KH, int KW, int H_pad, int W_pad, int H_stride, int W_stride, float prelu_alpha,
+                     float* d_y, void* stream) {
+    if (type < kTNN || type > kBNN) return fail(FTNN_EINVAL, "unknown network type %d", type);
+    int OH, OW;
+    int rc = check_conv_shape(N, C, H, W, H_pad, W_pad, KH, KW, H_stride, W_stride, &OH, &OW);
+    if (rc != FTNN_OK) return rc;
+    if (KN <= 0) return fail(FTNN_EINVAL, "non-positive kernel count");
+    const int64_t need = ftnn_conv_scratch_bytes(type, N, C, H, W, KN, KH, KW, H_pad, W_pad, H_stride, W_stride);
+    if (need <= 0 || need > kStaticScratchBytes)
+        return fail(FTNN_EINVAL, "layer needs %lld bytes of scratch, ftnn_conv_static holds %lld: use ftnn_conv with "
+                    "a buffer of the caller's", (long long)need, (long long)kStaticScratchBytes);
+    void* d_scr = static_scratch_of_current_device();
+    if (!d_scr) return FTNN_EHIP;
+    return ftnn_conv_engine(FTNN_ENGINE_AUTO, type, d_x, d_thr, d_qw, N, C, H, W, KN, KH, KW, H_pad, W_pad, H_stride,
+                            W_stride, prelu_alpha, d_scr, d_y, stream);
 }
 
 int ftnn_pack_weights(int ternary, const float* d_w, const float* d_thr, int KN, int C, int KH,

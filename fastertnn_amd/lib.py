@@ -42,6 +42,7 @@ _L.ftnn_mm_expanded.argtypes = [C.c_int, C.c_int, _vp, _vp] + [C.c_int] * 6 + [C
 _L.ftnn_conv_scratch_bytes.restype = C.c_int64
 _L.ftnn_conv_scratch_bytes.argtypes = [C.c_int] * 12
 _L.ftnn_conv.argtypes = [C.c_int, _vp, _vp, _vp] + [C.c_int] * 11 + [C.c_float, _vp, _vp, _vp]
+_L.ftnn_conv_static.argtypes = [C.c_int, _vp, _vp, _vp] + [C.c_int] * 11 + [C.c_float, _vp, _vp]
 _L.ftnn_conv_engine.argtypes = [C.c_int, C.c_int, _vp, _vp, _vp] + [C.c_int] * 11 + [C.c_float, _vp, _vp, _vp]
 _L.ftnn_select_conv_engine.argtypes = [C.c_int] * 12
 _L.ftnn_conv_weights_bytes.restype = C.c_int64
@@ -67,6 +68,7 @@ EXPORTS = ("tnns_conv", "tnns_gemm", "t2r_p2_opt", "b2r", "mm_tnn", "mm_tbn", "m
            "ftnn_pack_weights", "ftnn_pack_gemm_operand", "ftnn_select_engine", "ftnn_mm_scratch_bytes",
            "ftnn_mm_engine", "ftnn_expand_bytes", "ftnn_expand_rows", "ftnn_mm_expanded",
            "ftnn_conv_scratch_bytes", "ftnn_conv_engine", "ftnn_select_conv_engine",
+           "ftnn_conv_static",
            "ftnn_conv_weights_bytes", "ftnn_conv_prepare_weights", "ftnn_conv_prepared", "ftnn_net_create", "ftnn_net_create_ex", "ftnn_net_destroy", "ftnn_net_output_elems", "ftnn_net_run")
 
 ENGINE_AUTO, ENGINE_VALU, ENGINE_MFMA_I8, ENGINE_MFMA_F4 = 0, 1, 2, 3
@@ -207,6 +209,18 @@ def conv(typ, x, thr, qw, kn, kh, kw, pad, stride, alpha, scratch=None, out=None
     args = (typ, _dev(x, torch.float32), _dev(thr, torch.float32), _dev(qw), n, c, h, w, kn, kh, kw, pad, pad,
             stride, stride, alpha, _dev(scratch), _dev(out, torch.float32), _stream())
     _check(_L.ftnn_conv(*args) if engine == ENGINE_AUTO else _L.ftnn_conv_engine(engine, *args))
+    return out
+
+
+STATIC_SCRATCH_BYTES = 32 << 20
+
+
+def conv_static(typ, x, thr, qw, kn, kh, kw, pad, stride, alpha, out):
+    """ftnn_conv_static: the layer on the library's own fixed work space; allocates nothing (out is required)."""
+    import torch
+    n, c, h, w = x.shape
+    _check(_L.ftnn_conv_static(typ, _dev(x, torch.float32), _dev(thr, torch.float32), _dev(qw), n, c, h, w, kn, kh,
+                               kw, pad, pad, stride, stride, alpha, _dev(out, torch.float32), _stream()))
     return out
 
 

@@ -212,6 +212,22 @@ FTNN_API int ftnn_conv(int type, const float *d_x, const float *d_thr, const int
               int W_stride, float prelu_alpha, void *d_scratch, float *d_y, void *stream);
 
 /*
+ * ftnn_conv without a scratch argument and without any allocation.  No counterpart in the reference; it is for
+ * callers that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  The layer's work space (the quantised input and the weights in engine form) is a fixed array
+ * of FTNN_STATIC_SCRATCH_BYTES inside the library's code object, which every GPU the library runs on holds from
+ * the first call until the process ends.  A layer whose ftnn_conv_scratch_bytes() exceeds that is refused with
+ * FTNN_EINVAL.  The call itself performs no hipMalloc / hipFree and synchronises nothing; the first call on a
+ * device looks the array's address up (hipGetSymbolAddress), so make that first call outside a graph capture.
+ * All calls on one GPU share the one array: calls that overlap on a GPU (two streams, two threads) race, and the
+ * array keeps the last call's contents (every call overwrites the part it reads).  Same result as ftnn_conv.
+ */
+#define FTNN_STATIC_SCRATCH_BYTES (32 << 20)
+FTNN_API int ftnn_conv_static(int type, const float *d_x, const float *d_thr, const int64_t *d_qw, int N, int C,
+                              int H, int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride,
+                              int W_stride, float prelu_alpha, float *d_y, void *stream);
+
+/*
  * The same layer on an explicit engine (no counterpart in the reference; same bits on either):
  * FTNN_ENGINE_VALU      quantise to bit planes, vector-ALU popcount GEMM with implicit im2row;
  * FTNN_ENGINE_MFMA_F4   quantise to fp4 nibbles, expand the weights into matrix-core fragments
