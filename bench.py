@@ -2,19 +2,30 @@
 """Benchmark of the TNN hot path on one MI355X.
 
 Headline workload: the large compute-bound TNN GEMM (M = N = 8192, K = 32768,
-uniform ternary operands in Packing 2, PReLU(0.5) fused).  One "step" is one call
-of the GEMM entry point of the C ABI (`ftnn_mm`) with both packed operands and
-the output resident in HBM.  Prints ONE JSON line:
+uniform ternary operands in Packing 2, PReLU(0.5) fused).  One "step" is one pass of
+the GEMM over one batch of activation rows, everything resident in HBM: the packed
+activation operand A is turned into matrix-core fragments (ftnn_expand_rows) and
+multiplied with the weights B, which were brought into that form once before the timed
+region, as a layer keeps them (ftnn_mm_expanded).  Where the library's engine choice
+for the shape is the vector ALU the step is the one call ftnn_mm_engine.  Prints ONE
+JSON line:
 
-  value        ternary GMAC/s = M*N*K / time
-  roofline     vector-ALU roofline of the GEMM kernel: algorithmic lane-ops per
-               launch (4 VALU ops per pair of 32-lane dwords for TNN) over the
-               HIP-event duration of the launches, against 256 CU x 4 SIMD x 16
-               lanes x 2.4 GHz
+  value        ternary GMAC/s = M*N*K / time of a step
+  roofline     the dominant kernel of the step (the fp4 matrix-core GEMM): its launches
+               inside the timed region are bracketed by HIP events on the launch
+               stream; algorithmic FLOP per launch over their mean duration against
+               the published dense fp4 peak.  `traffic` comes from the tracked counter
+               summary under profiles/ (never a literal here).  Nested in it,
+               `valu_popcount`: the vector-ALU popcount kernel on the same operands
+               against 256 CU x 4 SIMD x 16 lanes x 2.4 GHz (the figure the metric
+               names), with the measured v_bcnt issue rate and the shader clocks of
+               probe and kernel, taken back to back in this process
   cpu_baseline the reference's own AVX2 GEMM (compiled from its sources into
                oracle/_ref) on one host core over a bounded row sample of the same
-               operands; the GPU rows of that sample are compared bit-for-bit
-  extra        conv-layer latencies (kernel-only and host-pointer ABI inclusive)
+               operands, or the AVX2 restatement under oracle/ where that build is
+               absent; the GPU rows of the sample are compared bit-for-bit
+  extra        conv-layer and layer-chain latencies (kernel-only and host-pointer ABI
+               inclusive); --full adds the reference's sweeps and tables
 """
 import argparse
 import json
@@ -41,6 +52,9 @@ def parse():
     ap.add_argument("--k", type=int, default=32768)
     ap.add_argument("--cpu-rows", type=int, default=8192, help="rows of A in the CPU-baseline sample (0 = skip)")
     ap.add_argument("--no-extra", action="store_true", help="skip the conv-layer latency section")
+    ap.add_argument("--full", action="store_true",
+                    help="also run the long sections (the reference's GEMM sweep, its 17 single layers and seven "
+                         "networks, other batch sizes and types); they go into the same JSON line under extra")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 256 MiB device copy, the known-size dispatch that "
                          "FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
@@ -85,23 +99,30 @@ def host_cpu():
 
 
 def cpu_gemm_baseline(a_host, b_host, rows, n, kw, alpha):
-    """reference mm_tnn on one core (its protocol pins the process to core 0, Makefile:21);
-    falls back to the plain-C port when the compiled reference is absent"""
+    """mm_tnn on ONE host core (the reference's protocol pins its drivers to core 0, Makefile:21): the reference's
+    own AVX2 path where its compiled form is present (kind "reference"), else the AVX2 restatement under oracle/
+    (kind "port"), else nothing -- the scalar oracle is a checker, not a baseline.  The affinity of the process is
+    restored afterwards.  Returns (y, seconds, kind) or (None, reason, None)."""
     from oracle import ftnn_oracle as O
-    try:
-        os.sched_setaffinity(0, {sorted(os.sched_getaffinity(0))[0]})
-    except (AttributeError, OSError):
-        pass
     if O.Reference.available():
-        ref, kind = O.Reference(), "reference"
-        t0 = time.perf_counter()
-        y = ref.mm(O.TNN, a_host, b_host, rows, 1, 1, n, kw, alpha)
-        dt = time.perf_counter() - t0
+        impl, kind = O.Reference(), "reference"
+    elif O.OracleAvx2.available():
+        impl, kind = O.OracleAvx2(), "port"
     else:
-        orc, kind = O.Oracle(), "port"
+        return None, "neither oracle/_ref/libref_final.so nor an AVX2 host: no CPU path of reference grade to time", None
+    saved = None
+    try:
+        saved = os.sched_getaffinity(0)
+        os.sched_setaffinity(0, {sorted(saved)[0]})
+    except (AttributeError, OSError):
+        saved = None
+    try:
         t0 = time.perf_counter()
-        y = orc.mm(O.TNN, a_host, b_host, rows, 1, 1, n, kw, alpha)
+        y = impl.mm(O.TNN, a_host, b_host, rows, 1, 1, n, kw, alpha)
         dt = time.perf_counter() - t0
+    finally:
+        if saved is not None:
+            os.sched_setaffinity(0, saved)
     return y, dt, kind
 
 
@@ -326,18 +347,85 @@ def e2e_latency(torch, lib, batch, reps=50, cpu=True, typ=None):
     return out
 
 
-def valu_probe():
-    """the measured issue rate of v_bcnt_u32_b32 over the whole chip (fastertnn_amd/csrc/probe_valu.hip, a child
-    process): what the nominal 39.3 T lane-op/s of the vector-ALU roofline comes to at the clock the chip holds"""
-    import subprocess
-    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fastertnn_amd", "probe_valu")
-    if not os.path.exists(exe):
-        return {"skipped": "fastertnn_amd/probe_valu is not built"}
-    p = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
-    for line in p.stdout.splitlines():
-        if line.startswith("{"):
-            return json.loads(line)
-    return {"failed": p.stdout[-200:]}
+class Probe:
+    """bench_probe/libprobe_valu.so: the v_bcnt issue-rate chain and the shader-clock sampler, run in this process on
+    torch's current stream"""
+
+    def __init__(self):
+        import ctypes as C
+        path = os.path.join(ROOT, "bench_probe", "libprobe_valu.so")
+        self.lib = C.CDLL(path) if os.path.exists(path) else None
+        self.C = C
+        if self.lib is not None and self.lib.probe_valu_init() != 0:
+            self.lib = None
+
+    def _call(self, fn, trips, torch, n):
+        out = (self.C.c_double * n)()
+        if fn(int(trips), self.C.c_void_p(torch.cuda.current_stream().cuda_stream), out) != 0:
+            return None
+        return list(out)
+
+    def copy(self, torch, src, dst):
+        out = (self.C.c_double * 1)()
+        rc = self.lib.probe_copy_run(self.C.c_void_p(src.data_ptr()), self.C.c_void_p(dst.data_ptr()),
+                                     self.C.c_size_t(src.numel() * src.element_size()),
+                                     self.C.c_void_p(torch.cuda.current_stream().cuda_stream), out)
+        return None if rc != 0 else out[0]
+
+    def issue_rate(self, torch, trips=2500):
+        r = self._call(self.lib.probe_valu_run, trips, torch, 5)
+        if r is None:
+            return None
+        return {"ms": round(r[0], 4), "lane_ops_per_s": float("%.4e" % r[1]), "frac_of_nominal": round(r[1] / (VALU_PEAK_TOPS * 1e12), 4),
+                "shader_mhz": round(r[2], 1), "lane_ops_per_lane_cycle": round(r[3], 4), "result_ok": bool(r[4])}
+
+    def clock_after(self, torch, trips=16):
+        """shader clock seen by a short, nearly idle kernel queued directly behind whatever ran last on the stream"""
+        r = self._call(self.lib.probe_clock_run, trips, torch, 2)
+        return None if r is None else {"ms": round(r[0], 4), "shader_mhz": round(r[1], 1)}
+
+
+def valu_reconciliation(torch, probe, run_valu, valu_ops, reps=12):
+    """The v_bcnt chain and the vector-ALU GEMM kernel back to back on one stream, with the shader clock each one
+    left behind (sampled by a 30 us kernel queued directly after it): the kernel's fraction of the NOMINAL roofline
+    (2.4 GHz) can exceed the probe's only when it ran at a higher clock, and its lane-ops per lane and cycle -- the
+    schedule-only figure -- is what compares like with like."""
+    if probe.lib is None:
+        return {"skipped": "bench_probe/libprobe_valu.so is not built"}
+    lanes = 256 * 4 * 16
+    out = {}
+    for _ in range(3):          # the same thermal / clock state for both: alternate them
+        probe.issue_rate(torch, 500)
+        run_valu()
+    p = probe.issue_rate(torch)
+    p["clock_after_mhz"] = (probe.clock_after(torch) or {}).get("shader_mhz")
+    out["probe"] = p
+    t = event_times(torch, run_valu, reps)
+    k_ms = sum(t) / len(t)
+    clk = probe.clock_after(torch)
+    out["kernel"] = {"avg_launch_ms": round(k_ms, 4), "frac_of_nominal": round(valu_ops / (k_ms * 1e-3) / 1e12 / VALU_PEAK_TOPS, 4),
+                     "clock_after_mhz": clk["shader_mhz"] if clk else None}
+    if clk and clk["shader_mhz"] > 0:
+        out["kernel"]["lane_ops_per_lane_cycle_at_that_clock"] = round(valu_ops / (k_ms * 1e-3) / (lanes * clk["shader_mhz"] * 1e6), 4)
+    p2 = probe.issue_rate(torch)
+    out["probe_again"] = {"frac_of_nominal": p2["frac_of_nominal"], "shader_mhz": p2["shader_mhz"],
+                          "lane_ops_per_lane_cycle": p2["lane_ops_per_lane_cycle"]}
+    return out
+
+
+def traffic_record(kernel_key, shape):
+    """HBM-side bytes per launch of `kernel_key` from the tracked counter summary profiles/traffic_*.json (written
+    by bench_probe/traffic_from_pmc.py from two rocprofv3 --pmc runs of this script); None when there is no record for
+    this shape"""
+    path = os.path.join(ROOT, "profiles", "traffic_tnn_gemm_%dx%dx%d.json" % shape)
+    try:
+        doc = json.load(open(path))
+        k = doc["kernels"][kernel_key]
+        return int(k["bytes_per_launch"]), {"file": os.path.relpath(path, ROOT), "commit": doc.get("commit"),
+                                            "date": doc.get("date"), "fetch_scale": doc.get("fetch_scale"),
+                                            "write_scale": doc.get("write_scale")}
+    except (OSError, KeyError, ValueError):
+        return None, None
 
 
 def reference_gemm_sweep(torch, lib, reps=10):
@@ -473,6 +561,39 @@ def reference_networks(torch, lib, batch=8, reps=5):
     return out
 
 
+def host_gemm_cfg4(torch, lib, a, b, m, n, kw, alpha=0.5):
+    """mm_tnn with host pointers on the headline shape (128 MiB in, 256 MiB out through PCIe): with the copy threads
+    the caller's CPU affinity allows, and pinned to one core as the reference's Makefile runs its drivers (then the
+    runtime's plain copies).  The library reads the affinity once, so each case runs in a child process."""
+    import subprocess
+    code = ("import sys, time, os, numpy as np\n"
+            "sys.path.insert(0, %r)\n"
+            "if sys.argv[1] == 'one': os.sched_setaffinity(0, {sorted(os.sched_getaffinity(0))[0]})\n"
+            "import fastertnn_amd.lib as lib\n"
+            "m, n, kw = %d, %d, %d\n"
+            "rng = np.random.default_rng(1)\n"
+            "def op(rows):\n"
+            "    r = rng.integers(0, 2 ** 63, size=(rows, kw // 4, 2, 4), dtype=np.int64)\n"
+            "    r[:, :, 0, :] &= ~r[:, :, 1, :]\n"
+            "    return r.reshape(-1)\n"
+            "a, b = op(m), op(n)\n"
+            "lib.host_mm(0, a, b, m, 1, 1, n, kw, 0.5)\n"
+            "t = []\n"
+            "for _ in range(3):\n"
+            "    t0 = time.perf_counter(); y = lib._L.mm_tnn(a.ctypes.data, b.ctypes.data, m, 1, 1, n, kw, 0.5); t.append(time.perf_counter() - t0); lib._libc.free(y)\n"
+            "print(min(t) * 1e3)\n" % (ROOT, m, n, kw))
+    out = {}
+    for mode in ("all", "one"):
+        try:
+            p = subprocess.run([sys.executable, "-c", code, mode], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+            ms = float(p.stdout.strip().splitlines()[-1])
+            out["caller_on_%s_core%s" % (mode, "s" if mode == "all" else "")] = {
+                "abi_ms": round(ms, 2), "gmacs_pcie_inclusive": round(float(m) * n * kw * 64 / ms / 1e6, 1)}
+        except Exception as e:   # noqa: BLE001 -- a failed side measurement must not lose the benchmark line
+            out["caller_on_%s_core%s" % (mode, "s" if mode == "all" else "")] = {"failed": str(e)[:200]}
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -495,14 +616,42 @@ def main():
     auto = lib.select_engine(TNN, m, 1, 1, n, kw)
     scratch = torch.empty(max(lib.mm_scratch_bytes(e, TNN, m, 1, 1, n, kw) for e in lib.ENGINE_NAMES) or 16,
                           dtype=torch.uint8, device="cuda")
+    macs = float(m) * n * k
 
-    def step():   # the timed hot path: packed operands in, fp32 result out, engine chosen by the library
-        lib.mm_engine(lib.ENGINE_AUTO, TNN, a, b, m, 1, 1, n, kw, alpha, out=y, scratch=scratch)
+    # The timed hot path.  Matrix-core engines: the weights B are in engine form already (done once, below, outside
+    # the timed region: a layer keeps its weights that way); a step expands the activation rows A and multiplies.
+    # The GEMM kernel of every timed step sits between two HIP events on the launch stream.
+    gemm_events = []
+    if auto == lib.ENGINE_VALU:
+        def step(timed=False):
+            if timed:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                gemm_events.append((e0, e1))
+                e0.record()
+            lib.mm_engine(lib.ENGINE_VALU, TNN, a, b, m, 1, 1, n, kw, alpha, out=y)
+            if timed:
+                e1.record()
+        step_desc = "ftnn_mm_engine (vector ALU) on the packed operands"
+    else:
+        b_exp = lib.expand_rows(auto, b, n, kw, True)
+        a_exp = torch.empty(int(lib._L.ftnn_expand_bytes(auto, m, kw)), dtype=torch.uint8, device="cuda")
+
+        def step(timed=False):
+            lib.expand_rows(auto, a, m, kw, True, out=a_exp)
+            if timed:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                gemm_events.append((e0, e1))
+                e0.record()
+            lib.mm_expanded(auto, TNN, a_exp, b_exp, m, 1, 1, n, kw, alpha, out=y)
+            if timed:
+                e1.record()
+        step_desc = ("ftnn_expand_rows(A) + ftnn_mm_expanded with B expanded once before the timed region "
+                     "(weights kept in engine form)")
 
     if args.copy_calibration:
         src = torch.empty(1 << 26, dtype=torch.float32, device="cuda").fill_(1.0)
         dst = torch.empty_like(src)
-        dst.copy_(src)
+        Probe().copy(torch, src, dst)    # k_probe_copy, 256 MiB each way
         torch.cuda.synchronize()
         del src, dst
 
@@ -511,17 +660,21 @@ def main():
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
+        step(timed=True)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
-    macs = float(m) * n * k
-    reps = min(max(args.steps, 5), 50)   # launches per event-timed mean below
+    gemm_ms = [e0.elapsed_time(e1) for e0, e1 in gemm_events]
+    gemm_avg = sum(gemm_ms) / len(gemm_ms)
+    y_step = y.clone()
 
     def mean(v):
         return sum(v) / len(v)
 
-    # every engine on the same operands, per-launch HIP events; the whole call (expansion included)
+    REPS = 30   # launches per event-timed mean in the sections below, whatever --steps says
+
+    # every engine on the same packed operands, per-launch HIP events: the whole call ftnn_mm_engine, both
+    # expansions included for the matrix-core engines
     engines = {}
     y_ref = None
     for eng, name in lib.ENGINE_NAMES.items():
@@ -532,46 +685,64 @@ def main():
         if y_ref is None:
             y_ref = y.clone()
         same = bool(torch.equal(y, y_ref))
-        t = mean(event_times(torch, run, reps))
+        t = mean(event_times(torch, run, REPS if name != "valu" else 12))
         engines[name] = {"call_ms": round(t, 4), "gmacs": round(macs / t / 1e6, 1), "same_bits_as_valu": same}
-    del y_ref
+    step_same = bool(torch.equal(y_step, y_ref))
+    del y_ref, y_step
 
-    # rooflines of the dominant kernels, each timed alone with HIP events on the launch stream
-    valu_ms = engines["valu"]["call_ms"]   # the VALU engine is one kernel
+    # the vector-ALU kernel against the roofline the metric names, with the issue-rate probe beside it
     valu_ops = 4.0 * m * n * (2 * kw)      # 4 vector ops per pair of 32-lane dwords, 2*kw dwords per plane
+    probe = Probe()
+
+    def run_valu():
+        lib.mm_engine(lib.ENGINE_VALU, TNN, a, b, m, 1, 1, n, kw, alpha, out=y)
+    recon = valu_reconciliation(torch, probe, run_valu, valu_ops)
+    valu_ms = recon["kernel"]["avg_launch_ms"] if "kernel" in recon else engines["valu"]["call_ms"]
     valu_ach = valu_ops / (valu_ms * 1e-3) / 1e12
+    traffic, traffic_src = traffic_record("k_mm", (m, n, k))
     roofline_valu = {"bound": "valu", "achieved": round(valu_ach, 3), "peak": round(VALU_PEAK_TOPS, 3),
-                     "unit": "Tlaneop/s", "frac": round(valu_ach / VALU_PEAK_TOPS, 4), "traffic": None,
-                     "kernel": "k_mm<TNN,2,8,1>", "avg_launch_ms": valu_ms,
+                     "unit": "Tlaneop/s", "frac": round(valu_ach / VALU_PEAK_TOPS, 4), "traffic": traffic,
+                     "kernel": "k_mm<TNN,2,8,1>", "avg_launch_ms": round(valu_ms, 4),
                      "popcount_frac": round(valu_ach / 2 / VALU_PEAK_TOPS, 4),
+                     "gmacs": round(macs / valu_ms / 1e6, 1),
+                     "probe_and_clocks": recon,
                      "note": "peak = 256 CU x 4 SIMD x 16 lanes x 2.4 GHz int32 VALU lane-ops; "
                              "algorithmic ops = 4 per dword pair (v_or, v_bitop3, 2 x v_bcnt)"}
     mfma = {}
-    for eng, kernel, peak in ((lib.ENGINE_MFMA_I8, "k_mfma<int8>", 5000.0), (lib.ENGINE_MFMA_F4, "k_mfma<fp4>", 10100.0)):
-        a_exp = lib.expand_rows(eng, a, m, kw, True)
-        b_exp = lib.expand_rows(eng, b, n, kw, True)
+    for eng, key, kernel, peak in ((lib.ENGINE_MFMA_I8, "k_mfma_i8", "k_mfma<int8>", 5000.0),
+                                   (lib.ENGINE_MFMA_F4, "k_mfma_f4", "k_mfma<fp4>", 10100.0)):
+        ae = lib.expand_rows(eng, a, m, kw, True)
+        be = lib.expand_rows(eng, b, n, kw, True)
 
-        def gemm(eng=eng, a_exp=a_exp, b_exp=b_exp):
-            lib.mm_expanded(eng, TNN, a_exp, b_exp, m, 1, 1, n, kw, alpha, out=y)
+        def gemm(eng=eng, ae=ae, be=be):
+            lib.mm_expanded(eng, TNN, ae, be, m, 1, 1, n, kw, alpha, out=y)
 
-        def expand(eng=eng, a_exp=a_exp):
-            lib.expand_rows(eng, a, m, kw, True, out=a_exp)
+        def expand(eng=eng, ae=ae):
+            lib.expand_rows(eng, a, m, kw, True, out=ae)
         gemm()
-        t = mean(event_times(torch, gemm, reps))
-        te = mean(event_times(torch, expand, reps))
+        t = mean(event_times(torch, gemm, REPS))
+        te = mean(event_times(torch, expand, REPS))
+        if eng == auto:
+            t = gemm_avg          # the headline kernel: its launches inside the timed region
         ach = 2.0 * macs / (t * 1e-3) / 1e12
+        traffic, src = traffic_record(key, (m, n, k))
         mfma[eng] = {"bound": "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "TOP/s" if eng == lib.ENGINE_MFMA_I8 else "TFLOP/s",
-                     "frac": round(ach / peak, 4), "traffic": None, "kernel": kernel, "avg_launch_ms": round(t, 4),
+                     "frac": round(ach / peak, 4), "traffic": traffic, "kernel": kernel, "avg_launch_ms": round(t, 4),
                      "expand_one_operand_ms": round(te, 4)}
-        del a_exp, b_exp
-    if (m, n, k) == (8192, 8192, 32768):
-        # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE (KiB per dispatch, scaled by a plain 256 MiB
-        # copy: x2.0 / x1.0), measured with this script under the profiler: profiles/tnn_gemm_8192x8192x32768_all_engines.md
-        roofline_valu["traffic"] = int((2049521.1 * 2.0 + 262183.5) * 1024)
-        mfma[lib.ENGINE_MFMA_I8]["traffic"] = int((1574007.8 * 2.0 + 262144.0) * 1024)
-        mfma[lib.ENGINE_MFMA_F4]["traffic"] = int((790714.8 * 2.0 + 262144.0) * 1024)
-    roofline = {lib.ENGINE_VALU: roofline_valu, lib.ENGINE_MFMA_I8: mfma[lib.ENGINE_MFMA_I8],
-                lib.ENGINE_MFMA_F4: mfma[lib.ENGINE_MFMA_F4]}[auto]
+        if eng == auto:
+            mfma[eng]["launches_timed"] = len(gemm_ms)
+            mfma[eng]["timed"] = "HIP events around each GEMM launch of the timed region"
+            mfma[eng]["traffic_source"] = src
+        del ae, be
+    if auto == lib.ENGINE_VALU:
+        roofline = dict(roofline_valu)
+    else:
+        roofline = dict(mfma[auto])
+        roofline["valu_popcount"] = {"frac": roofline_valu["frac"], "popcount_frac": roofline_valu["popcount_frac"],
+                                     "achieved": roofline_valu["achieved"], "peak": roofline_valu["peak"], "unit": "Tlaneop/s",
+                                     "avg_launch_ms": roofline_valu["avg_launch_ms"], "kernel": roofline_valu["kernel"],
+                                     "gmacs": roofline_valu["gmacs"], "traffic": roofline_valu["traffic"],
+                                     "probe_and_clocks": recon}
 
     cpu = None
     if args.cpu_rows > 0:
@@ -580,31 +751,39 @@ def main():
         b_host = b.cpu().numpy()
         from oracle.ftnn_oracle import aligned_copy
         y_cpu, dt, kind = cpu_gemm_baseline(aligned_copy(a_host), aligned_copy(b_host), rows, n, kw, alpha)
-        y_gpu = y.view(m, n)[:rows].cpu().numpy()
-        cpu = {"value": round(float(rows) * n * k / dt / 1e9, 2), "unit": "GMAC/s", "cores": 1, "kind": kind,
-               "sample": "first %d of %d rows of A against all %d columns, K=%d (%.1f s on one core)"
-                         % (rows, m, n, k, dt),
-               "gpu_rows_bit_exact": bool(y_gpu.tobytes() == np.ascontiguousarray(y_cpu).tobytes()),
-               "host": host_cpu()}
+        if y_cpu is None:
+            cpu = {"value": None, "reason": dt}
+        else:
+            step()
+            torch.cuda.synchronize()
+            y_gpu = y.view(m, n)[:rows].cpu().numpy()
+            cpu = {"value": round(float(rows) * n * k / dt / 1e9, 2), "unit": "GMAC/s", "cores": 1, "kind": kind,
+                   "sample": "first %d of %d rows of A against all %d columns, K=%d (%.1f s on one core)"
+                             % (rows, m, n, k, dt),
+                   "gpu_rows_bit_exact": bool(y_gpu.tobytes() == np.ascontiguousarray(y_cpu).tobytes()),
+                   "host": host_cpu()}
 
     extra = None
     if not args.no_extra:
         extra = {
-            "other_types_same_gemm_shape": other_types(torch, lib, a, b, m, n, k),
             "tnn_gemm_256x256x4096": small_gemm(torch, lib, 256, 256, 4096),
-            "quantize_im2row_pack": pack_rates(torch, lib),
             "tnn_conv_b1_c256_56x56_k3": conv_latency(torch, lib, TNN, (256, 56, 56, 256, 3, 3, 1, 1), 1, 2),
             "tbn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, TBN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 3),
             "btn_conv_b8_c128_28x28_k3": conv_latency(torch, lib, BTN, (128, 28, 28, 128, 3, 3, 1, 1), 8, 4),
             "tnn_resnet18_like_b32_e2e": e2e_latency(torch, lib, 32),
-            "valu_popcount_probe": valu_probe(),
-            "reference_gemm_sweep": reference_gemm_sweep(torch, lib),
-            "reference_single_layers_b8": reference_single_layers(torch, lib),
-            "reference_e2e_networks_b8": reference_networks(torch, lib),
-            "tnn_resnet18_like_other_batches": {"b%d" % b: e2e_latency(torch, lib, b, cpu=False) for b in (1, 8, 128)},
-            "other_types_resnet18_like_b32": {n: e2e_latency(torch, lib, 32, cpu=False, typ=t)
-                                              for n, t in (("tbn", 1), ("btn", 2), ("bnn", 3))},
+            "quantize_im2row_pack": pack_rates(torch, lib),
+            "host_mm_8192x8192x32768": host_gemm_cfg4(torch, lib, a, b, m, n, kw) if (m, n, k) == (8192, 8192, 32768) else None,
         }
+        if args.full:
+            extra.update({
+                "other_types_same_gemm_shape": other_types(torch, lib, a, b, m, n, k),
+                "reference_gemm_sweep": reference_gemm_sweep(torch, lib),
+                "reference_single_layers_b8": reference_single_layers(torch, lib),
+                "reference_e2e_networks_b8": reference_networks(torch, lib),
+                "tnn_resnet18_like_other_batches": {"b%d" % bb: e2e_latency(torch, lib, bb, cpu=False) for bb in (1, 8, 128)},
+                "other_types_resnet18_like_b32": {nm: e2e_latency(torch, lib, 32, cpu=False, typ=t)
+                                                  for nm, t in (("tbn", 1), ("btn", 2), ("bnn", 3))},
+            })
 
     line = {
         "metric": "TNN GEMM ternary GMAC/s", "value": round(macs / (ms_per_step * 1e-3) / 1e9, 1),
@@ -612,11 +791,12 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": {1: "u32", 2: "int8", 3: "fp4 (E2M1, exact for -1/0/+1) with fp32 accumulate"}[auto], "data": "synthetic",
         "config": {"workload": "TNN GEMM M=%d N=%d K=%d, uniform ternary, Packing 2, PReLU 0.5 fused" % (m, n, k),
-                   "m": m, "n": n, "k": k},
+                   "m": m, "n": n, "k": k, "step": step_desc},
         "roofline": roofline, "cpu_baseline": cpu,
-        "engine": lib.ENGINE_NAMES[auto], "engines": engines,
-        "roofline_valu_kernel": roofline_valu, "roofline_mfma_i8_kernel": mfma[lib.ENGINE_MFMA_I8],
-        "roofline_mfma_f4_kernel": mfma[lib.ENGINE_MFMA_F4], "extra": extra,
+        "engine": lib.ENGINE_NAMES[auto], "step_same_bits_as_valu": step_same,
+        "engines_whole_call_from_packed_operands": engines,
+        "roofline_mfma_i8_kernel": mfma[lib.ENGINE_MFMA_I8] if auto != lib.ENGINE_MFMA_I8 else None,
+        "extra": extra,
     }
     print(json.dumps(line), flush=True)
 

@@ -1,0 +1,171 @@
+// Measurement aid of bench.py (its own small shared library, not part of libftnn_hip.so): the vector-ALU issue
+// rate the popcount GEMM is priced against, and the shader clock the chip holds while it runs.
+//
+//   probe_valu_run    every wavefront of a chip-filling grid runs a long chain of v_bcnt_u32_b32 (population count
+//                     with accumulate) on independent registers, nothing else in the loop but the counter.  The
+//                     first wavefront of every workgroup also reads the shader-clock counter (s_memtime) and the
+//                     constant-rate counter (s_memrealtime) before and after its loop: their ratio is the shader
+//                     clock that kernel really ran at, which is what turns "lane-ops per second" into "lane-ops
+//                     per cycle".
+//   probe_clock_run   a short, nearly idle kernel (one wavefront per compute unit, the same chain for a few tens
+//                     of microseconds) that only reports that clock ratio: queued directly behind another kernel
+//                     on the same stream it samples the clock that kernel left the chip at.
+//
+//   probe_copy_run    a plain copy kernel of known size (k_probe_copy: 16 bytes per thread in, 16 bytes out): the
+//                     dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by.
+//
+// All are launched on the caller's stream and timed with HIP events recorded on that stream.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+
+namespace {
+
+constexpr int kAcc = 8;      // independent accumulators per lane
+constexpr int kUnroll = 64;  // popcounts per accumulator and loop trip: 512 vector instructions per 3 scalar ones of loop control
+
+struct Stamp {
+    unsigned long long clk0, clk1, rt0, rt1;
+};
+
+__global__ __launch_bounds__(256) void k_bcnt(const uint32_t* __restrict__ in, uint32_t* __restrict__ out, int trips,
+                                              Stamp* __restrict__ stamps) {
+    uint32_t x[kAcc], acc[kAcc];
+#pragma unroll
+    for (int i = 0; i < kAcc; i++) {
+        x[i] = in[(threadIdx.x + 64 * i) & 1023];
+        acc[i] = 0;
+    }
+    const unsigned long long c0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+    for (int t = 0; t < trips; t++) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++)
+#pragma unroll
+            for (int i = 0; i < kAcc; i++) asm volatile("v_bcnt_u32_b32 %0, %1, %0" : "+v"(acc[i]) : "v"(x[i]));
+    }
+    const unsigned long long c1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
+    uint32_t s = 0;
+#pragma unroll
+    for (int i = 0; i < kAcc; i++) s += acc[i];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+    if (threadIdx.x == 0) stamps[blockIdx.x] = Stamp{c0, c1, r0, r1};
+}
+
+__global__ __launch_bounds__(256) void k_probe_copy(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n16) dst[i] = src[i];
+}
+
+struct State {
+    uint32_t *in = nullptr, *out = nullptr;
+    Stamp *stamps = nullptr, *stamps_host = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    int cus = 0, blocks = 0;
+    double realtime_hz = 1e8;
+    uint32_t host_in[1024];
+} g;
+
+bool ok(hipError_t e, const char* what) {
+    if (e != hipSuccess) fprintf(stderr, "probe_valu: %s: %s\n", what, hipGetErrorString(e));
+    return e == hipSuccess;
+}
+
+// mean shader clock in MHz over the workgroups' stamps
+double mean_mhz(int blocks) {
+    double sum = 0.0;
+    int n = 0;
+    for (int b = 0; b < blocks; b++) {
+        const Stamp& s = g.stamps_host[b];
+        if (s.rt1 > s.rt0) {
+            sum += (double)(s.clk1 - s.clk0) / ((double)(s.rt1 - s.rt0) / g.realtime_hz) / 1e6;
+            n++;
+        }
+    }
+    return n ? sum / n : 0.0;
+}
+
+}  // namespace
+
+extern "C" {
+
+// allocates the probe's buffers on the current device; 0 on success
+__attribute__((visibility("default"))) int probe_valu_init(void) {
+    if (g.in) return 0;
+    hipDeviceProp_t prop;
+    if (!ok(hipGetDeviceProperties(&prop, 0), "hipGetDeviceProperties")) return 1;
+    g.cus = prop.multiProcessorCount;
+    g.blocks = g.cus * 8;   // 8 workgroups of 4 wavefronts per compute unit: 8 wavefronts per SIMD
+    int khz = 0;
+    if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, 0) == hipSuccess && khz > 0) g.realtime_hz = khz * 1e3;
+    if (!ok(hipMalloc(&g.in, sizeof g.host_in), "hipMalloc") ||
+        !ok(hipMalloc(&g.out, (size_t)g.blocks * 256 * 4), "hipMalloc") ||
+        !ok(hipMalloc(&g.stamps, (size_t)g.blocks * sizeof(Stamp)), "hipMalloc") ||
+        !ok(hipHostMalloc((void**)&g.stamps_host, (size_t)g.blocks * sizeof(Stamp), hipHostMallocDefault), "hipHostMalloc"))
+        return 1;
+    for (int i = 0; i < 1024; i++) g.host_in[i] = 0x9E3779B9u * (uint32_t)(i + 1);
+    if (!ok(hipMemcpy(g.in, g.host_in, sizeof g.host_in, hipMemcpyHostToDevice), "hipMemcpy")) return 1;
+    if (!ok(hipEventCreate(&g.e0), "hipEventCreate") || !ok(hipEventCreate(&g.e1), "hipEventCreate")) return 1;
+    return 0;
+}
+
+__attribute__((visibility("default"))) int probe_valu_compute_units(void) { return g.cus; }
+
+// The chip-filling chain.  out[0] = kernel ms (HIP events on `stream`), out[1] = lane-ops per second,
+// out[2] = mean shader clock in MHz during the kernel, out[3] = lane-ops per lane and cycle at that clock
+// (1.0 = one vector instruction per cycle and SIMD), out[4] = 1 if the accumulated counts are right.
+__attribute__((visibility("default"))) int probe_valu_run(int trips, void* stream, double* out) {
+    if (probe_valu_init() != 0) return 1;
+    hipStream_t st = (hipStream_t)stream;
+    if (!ok(hipEventRecord(g.e0, st), "hipEventRecord")) return 1;
+    hipLaunchKernelGGL(k_bcnt, dim3(g.blocks), dim3(256), 0, st, g.in, g.out, trips, g.stamps);
+    if (!ok(hipGetLastError(), "launch") || !ok(hipEventRecord(g.e1, st), "hipEventRecord")) return 1;
+    if (!ok(hipMemcpyAsync(g.stamps_host, g.stamps, (size_t)g.blocks * sizeof(Stamp), hipMemcpyDeviceToHost, st), "copy")) return 1;
+    uint32_t got = 0;
+    if (!ok(hipMemcpyAsync(&got, g.out, 4, hipMemcpyDeviceToHost, st), "copy") || !ok(hipStreamSynchronize(st), "sync")) return 1;
+    float ms = 0.0f;
+    if (!ok(hipEventElapsedTime(&ms, g.e0, g.e1), "hipEventElapsedTime")) return 1;
+    uint32_t want = 0;
+    for (int i = 0; i < kAcc; i++) want += (uint32_t)trips * kUnroll * (uint32_t)__builtin_popcount(g.host_in[(64 * i) & 1023]);
+    const double lane_ops = (double)g.blocks * 256 * trips * kUnroll * kAcc;
+    out[0] = ms;
+    out[1] = lane_ops / (ms * 1e-3);
+    out[2] = mean_mhz(g.blocks);
+    out[3] = out[2] > 0 ? out[1] / ((double)g.cus * 4 * 16 * out[2] * 1e6) : 0.0;
+    out[4] = got == want ? 1.0 : 0.0;
+    return 0;
+}
+
+// One wavefront per compute unit for `trips` loop trips: out[0] = kernel ms, out[1] = mean shader clock in MHz.
+__attribute__((visibility("default"))) int probe_clock_run(int trips, void* stream, double* out) {
+    if (probe_valu_init() != 0) return 1;
+    hipStream_t st = (hipStream_t)stream;
+    if (!ok(hipEventRecord(g.e0, st), "hipEventRecord")) return 1;
+    hipLaunchKernelGGL(k_bcnt, dim3(g.cus), dim3(64), 0, st, g.in, g.out, trips, g.stamps);
+    if (!ok(hipGetLastError(), "launch") || !ok(hipEventRecord(g.e1, st), "hipEventRecord")) return 1;
+    if (!ok(hipMemcpyAsync(g.stamps_host, g.stamps, (size_t)g.cus * sizeof(Stamp), hipMemcpyDeviceToHost, st), "copy") ||
+        !ok(hipStreamSynchronize(st), "sync"))
+        return 1;
+    float ms = 0.0f;
+    if (!ok(hipEventElapsedTime(&ms, g.e0, g.e1), "hipEventElapsedTime")) return 1;
+    out[0] = ms;
+    out[1] = mean_mhz(g.cus);
+    return 0;
+}
+
+// Copies `bytes` (a multiple of 4096) from d_src to d_dst with k_probe_copy; out[0] = kernel ms.
+__attribute__((visibility("default"))) int probe_copy_run(const void* d_src, void* d_dst, size_t bytes, void* stream, double* out) {
+    if (probe_valu_init() != 0 || bytes % 4096 != 0 || bytes / 4096 > 0x7fffffffull) return 1;
+    hipStream_t st = (hipStream_t)stream;
+    if (!ok(hipEventRecord(g.e0, st), "hipEventRecord")) return 1;
+    hipLaunchKernelGGL(k_probe_copy, dim3((unsigned)(bytes / 4096)), dim3(256), 0, st, static_cast<const uint4*>(d_src),
+                       static_cast<uint4*>(d_dst), bytes / 16);
+    if (!ok(hipGetLastError(), "launch") || !ok(hipEventRecord(g.e1, st), "hipEventRecord") || !ok(hipStreamSynchronize(st), "sync"))
+        return 1;
+    float ms = 0.0f;
+    if (!ok(hipEventElapsedTime(&ms, g.e0, g.e1), "hipEventElapsedTime")) return 1;
+    out[0] = ms;
+    return 0;
+}
+
+}  // extern "C"

@@ -6,7 +6,6 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libftnn_hip.so")
-PROBE = os.path.join(HERE, "probe_valu")   # stand-alone measurement aid (vector-ALU popcount issue rate)
 SOURCES = ["ftnn_api.hip", "pack_kernels.hip", "mm_kernels.hip", "mfma_kernels.hip", "stem_kernels.hip", "ftnn_net.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
@@ -14,25 +13,30 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hi
          "-Wall", "-Wno-unused-function"]
 
 
-# Kernels that issue loads through inline asm and count them by hand: a register of theirs that the compiler
-# keeps in scratch memory could be the target of a load in flight, so the build refuses scratch use in them
-# (the library checks the same at run time before the first launch).
-NO_SCRATCH = {"mfma_kernels.hip": "k_conv_f4"}
+# Kernels that issue loads through inline asm and count them by hand (s_waitcnt vmcnt(N)): a register of theirs
+# that the compiler keeps in scratch memory could be the target of a load in flight, and every scratch access is
+# itself a vector-memory operation that moves the count the waits rely on.  The build refuses scratch use in
+# them (the library checks the same at run time before the first launch).  Source -> name fragments.
+NO_SCRATCH = {"mfma_kernels.hip": ("k_conv_f4", "k_mfma")}
 
 
 def check_no_scratch(src, remarks):
     """parse -Rpass-analysis=kernel-resource-usage remarks; raise if a listed kernel uses scratch"""
-    name, bad, seen = None, [], 0
+    name, bad, seen = None, [], {frag: 0 for frag in NO_SCRATCH[src]}
     for line in remarks.splitlines():
         if "remark: Function Name:" in line:
             name = line.split("Function Name:")[1].split()[0]
-        elif "ScratchSize [bytes/lane]:" in line and name and NO_SCRATCH[src] in name:
-            seen += 1
-            if int(line.split("ScratchSize [bytes/lane]:")[1].split()[0]) != 0:
-                bad.append(name)
-    if bad or not seen:
+        elif "ScratchSize [bytes/lane]:" in line and name:
+            for frag in NO_SCRATCH[src]:
+                if frag in name:
+                    seen[frag] += 1
+                    if int(line.split("ScratchSize [bytes/lane]:")[1].split()[0]) != 0:
+                        bad.append(name)
+                    break
+    missing = [frag for frag, n in seen.items() if n == 0]
+    if bad or missing:
         raise RuntimeError("%s: %s" % (src, "kernels with scratch memory: %s" % bad if bad else
-                                       "no resource remarks found for %s" % NO_SCRATCH[src]))
+                                       "no resource remarks found for %s" % missing))
 
 
 def build_library(verbose=False):
@@ -61,18 +65,7 @@ def build_library(verbose=False):
             print(out)
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB]
     subprocess.run(cmd, check=True)
-    build_probe()
     return LIB
-
-
-def build_probe():
-    """the popcount issue-rate probe bench.py runs beside the GEMM (its own executable, not part of the library)"""
-    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-           "-packed-fp32-ops", os.path.join(CSRC, "probe_valu.hip"), "-o", PROBE]
-    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if p.returncode != 0:
-        raise RuntimeError("hipcc failed on probe_valu.hip:\n%s" % p.stdout)
-    return PROBE
 
 
 if __name__ == "__main__":

@@ -761,8 +761,16 @@ hipError_t launch_gemm_tile(const uint4* Pf, const uint4* Qf, float* Y, int M, i
     auto kern = k_mfma<F4, SWAP, WT, KF, NS>;
     constexpr size_t lds_bytes = Tile<WT, KF, NS>::lds_bytes;
     // the opt-in to more than 64 KiB of dynamic LDS is per kernel; done once, thread-safe
-    static const hipError_t configured = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    // The kernel counts its LDS-direct loads by hand (s_waitcnt vmcnt(N)); a scratch access would be one more
+    // vector-memory operation inside those windows, so a build of it that spills is refused (once per variant).
+    static const hipError_t configured = []() {
+        const void* kern = reinterpret_cast<const void*>(&k_mfma<F4, SWAP, WT, KF, NS>);
+        hipFuncAttributes attr;
+        hipError_t e = hipFuncGetAttributes(&attr, kern);
+        if (e == hipSuccess && attr.localSizeBytes != 0) e = hipErrorLaunchFailure;
+        if (e != hipSuccess) return e;
+        return hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)Tile<WT, KF, NS>::lds_bytes);
+    }();
     if (configured != hipSuccess) return configured;
     const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN, edge = 64 * WT;
     dim3 grid((prow + edge - 1) / edge, (qrow + edge - 1) / edge);
@@ -838,8 +846,12 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
     const int64_t tiles = ((M + 63) / 64) * ((KN + 63) / 64);
     int split = tiles >= 600 ? 1 : (tiles >= 450 ? 2 : 4);   // measured on MI355X (1024 SIMDs)
     while (split > 1 && cg.K < split) split /= 2;   // no wavefront without K words of its own
-    static const char* tune = getenv("FTNN_CONV_SPLIT");   // tuning aid: force the K split
-    if (tune) split = atoi(tune);
+    static const int tune = []() {   // tuning aid: force the K split (1, 2 or 4; anything else is ignored)
+        const char* e = getenv("FTNN_CONV_SPLIT");
+        const int v = e ? atoi(e) : 0;
+        return (v == 1 || v == 2 || v == 4) ? v : 0;
+    }();
+    if (tune) split = tune;
     const int wpb = 4, tpb = wpb / split;   // wavefronts and pixel tiles per workgroup (see the kernel)
     // few 64 x 64 tiles: tiles of 32 x 32, four times the workgroups (k_conv_f4_small)
     static const int small_below = getenv("FTNN_CONV_SMALL_BELOW") ? atoi(getenv("FTNN_CONV_SMALL_BELOW")) : 150;

@@ -15,7 +15,9 @@
 //
 // Weights (ternarize_opt_avx2 / binarize_opt_avx2, src/utils.c:468-521,634-675)
 // and GEMM operands (bitpacking2, src/utils.c:257-291) are packed by their own
-// kernels; they are offline work in the reference and are not tuned here.
+// ballot kernels (k_pack_weights, k_pack_gemm_operand): offline work in the
+// reference, HBM-bound here (a wavefront per output word group, several coalesced
+// loads in flight per lane).
 #include "ftnn_internal.h"
 
 namespace ftnn {

@@ -3,6 +3,9 @@
 Three libraries are bound here:
 
 * ``Oracle``     -- ``libftnn_oracle.so``, the plain-C restatement in this directory.
+* ``OracleAvx2`` -- ``libftnn_oracle_avx2.so``, the TNN GEMM restated with AVX2 intrinsics
+  (the reference's blocking and popcount scheme): the benchmark's CPU baseline where the
+  compiled reference is absent.
 * ``Reference``  -- ``_ref/libref_final.so``, the reference's own AVX2 "final" path
   compiled from its sources (present only where ``make ref`` ran or its output
   was carried along).  It validates the restatement, writes the golden vectors
@@ -21,6 +24,7 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ORACLE_SO = os.path.join(HERE, "libftnn_oracle.so")
+ORACLE_AVX2_SO = os.path.join(HERE, "libftnn_oracle_avx2.so")
 REF_SO = os.path.join(HERE, "_ref", "libref_final.so")
 REF_BASELINE_SO = os.path.join(HERE, "_ref", "libref_baseline.so")
 
@@ -142,6 +146,29 @@ class Oracle:
     def gemm(self, xp, wp, m, n, p_packed):
         y = np.empty((m, n), dtype=np.float32)
         self.lib.orc_tnns_gemm(_p(xp, _i64p), _p(wp, _i64p), m, n, p_packed, _p(y, _f32p))
+        return y
+
+
+class OracleAvx2:
+    """orc_avx2_mm_tnn: needs a CPU with AVX2 and 32-byte aligned operands (aligned_copy)"""
+
+    @staticmethod
+    def available():
+        try:
+            flags = next(l for l in open("/proc/cpuinfo") if l.startswith("flags"))
+        except (OSError, StopIteration):
+            return False
+        return " avx2" in flags and os.path.exists(ORACLE_AVX2_SO)
+
+    def __init__(self, path=ORACLE_AVX2_SO):
+        self.lib = C.CDLL(path)
+        self.lib.orc_avx2_mm_tnn.restype = None
+
+    def mm(self, typ, a, b, n, oh, ow, kn, k, alpha, k_unpack=0):
+        assert typ == TNN, "the AVX2 restatement covers the TNN GEMM"
+        assert a.ctypes.data % 32 == 0 and b.ctypes.data % 32 == 0
+        y = np.empty(n * kn * oh * ow, dtype=np.float32)
+        self.lib.orc_avx2_mm_tnn(_p(a, _i64p), _p(b, _i64p), n, oh, ow, kn, k, C.c_float(alpha), _p(y, _f32p))
         return y
 
 

@@ -146,20 +146,33 @@ def test_build_refuses_scratch_in_hand_counted_kernels():
     ok = ("x.hip:1:1: remark: Function Name: _ZN4ftnn9k_conv_f4ILb0EEEvv [-Rpass-analysis=kernel-resource-usage]\n"
           "x.hip:1:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]\n"
           "x.hip:1:1: remark: Function Name: _ZN4ftnn6k_mfmaEvv [-Rpass-analysis=kernel-resource-usage]\n"
+          "x.hip:1:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]\n"
+          "x.hip:1:1: remark: Function Name: _ZN4ftnn8k_expandEvv [-Rpass-analysis=kernel-resource-usage]\n"
           "x.hip:1:1: remark:     ScratchSize [bytes/lane]: 64 [-Rpass-analysis=kernel-resource-usage]\n")
-    build.check_no_scratch("mfma_kernels.hip", ok)
-    with pytest.raises(RuntimeError, match="scratch"):
-        build.check_no_scratch("mfma_kernels.hip", ok.replace("lane]: 0", "lane]: 60"))
+    build.check_no_scratch("mfma_kernels.hip", ok)   # scratch in a kernel that counts nothing by hand is no error
+    for kernel in ("k_conv_f4", "k_mfma"):           # in either hand-counted kernel it is
+        lines = ok.splitlines(True)
+        at = next(i for i, l in enumerate(lines) if kernel in l)
+        lines[at + 1] = lines[at + 1].replace("lane]: 0", "lane]: 60")
+        with pytest.raises(RuntimeError, match="scratch"):
+            build.check_no_scratch("mfma_kernels.hip", "".join(lines))
     with pytest.raises(RuntimeError, match="no resource remarks"):
         build.check_no_scratch("mfma_kernels.hip", "")
+    with pytest.raises(RuntimeError, match="k_mfma"):   # remarks for one of the two only
+        build.check_no_scratch("mfma_kernels.hip", "".join(ok.splitlines(True)[:2]))
 
 
-def test_popcount_probe_is_built_beside_the_library():
-    """bench.py runs it as a child process for the measured vector-ALU issue rate"""
+def test_benchmark_probe_is_built_outside_the_library():
+    """bench.py loads it for the measured vector-ALU issue rate; it is no part of the shipped package"""
+    import ctypes
     import os
+    from bench_probe import build as probe_build
     from fastertnn_amd import build
-    assert os.path.exists(build.LIB)
-    assert os.access(build.PROBE, os.X_OK)
+    assert os.path.exists(build.LIB) and os.path.exists(probe_build.LIB)
+    dll = ctypes.CDLL(probe_build.LIB)
+    for name in ("probe_valu_init", "probe_valu_run", "probe_clock_run"):
+        assert hasattr(dll, name)
+    assert not os.path.exists(os.path.join(os.path.dirname(build.LIB), "probe_valu"))
 
 
 def test_size_limits_need_no_device():
