@@ -16,7 +16,9 @@ DRIVER = os.path.join(ROOT, "oracle", "_ref", "ref_timing_layers")
 @pytest.mark.parametrize("net", ["tnn", "tbn", "btn", "bnn"])
 def test_reference_driver_self_test_passes_on_the_hip_library(net, tmp_path):
     if not os.path.exists(DRIVER):
-        pytest.skip("oracle/_ref/ref_timing_layers not present (built only where the reference tree is)")
+        pytest.skip("NOT RUN: oracle/_ref/ref_timing_layers is absent (it is compiled from the reference tree, which "
+                    "this machine lacks, and travels as a built file); tests/test_gpu_harness.py runs the same 12 "
+                    "shapes through the repository's own driver")
     os.makedirs(tmp_path / "out" / "measurements")
     print("case reference driver", net, flush=True)
     r = subprocess.run([DRIVER, "final", net, "test"], cwd=str(tmp_path), capture_output=True, text=True,
