@@ -4,7 +4,10 @@
 #include <stdio.h>
 
 #include <sched.h>
+#include <malloc.h>
 #include <stdlib.h>
+#include <sys/mman.h>
+#include <time.h>
 #include <string.h>
 
 #include <algorithm>
@@ -84,8 +87,30 @@ static void hip_or_die(hipError_t e, const char* what) {
     }
 }
 
+// Every host entry point returns a buffer that the caller free()s, call after call, layer after layer.  With the
+// allocator's defaults such buffers are cut from the top of the heap and given back to the system as soon as 2 x the
+// largest of them is free there, or are mappings of their own beyond 32 MiB: a good part of the results then lands in
+// memory that has to be faulted in again, page by page, by the copy (ResNet-152 through the reference's e2e driver:
+// five results of 25 MB per pass at 4.4 ms instead of 0.6 ms each).  With FTNN_HOST_KEEP_HEAP=1 in the environment the
+// host entry points tell the allocator on their first call to keep freed memory (blocks up to 32 MiB from the heap,
+// the heap's top trimmed only beyond 512 MiB): 163 -> 155 ms on that network, 24 -> 21 ms on VGG-16.  Off by default:
+// it changes the allocator of the whole process.
+static void keep_heap_once() {
+    static const bool done = []() {
+        const char* e = getenv("FTNN_HOST_KEEP_HEAP");
+        if (!e || atoi(e) == 0) return true;
+        mallopt(M_MMAP_THRESHOLD, 32 << 20);
+        mallopt(M_TRIM_THRESHOLD, 512 << 20);
+        return true;
+    }();
+    (void)done;
+}
+
 static hipStream_t host_stream() {
-    if (!g_ctx.stream) hip_or_die(hipStreamCreate(&g_ctx.stream), "hipStreamCreate");
+    if (!g_ctx.stream) {
+        keep_heap_once();
+        hip_or_die(hipStreamCreate(&g_ctx.stream), "hipStreamCreate");
+    }
     return g_ctx.stream;
 }
 
@@ -112,7 +137,7 @@ static void* dev_buf(int slot, size_t bytes) {
 // the copies here go through a small ring of pinned chunks instead: the DMA engine moves a chunk (57 GB/s) while
 // a few threads copy the neighbouring chunk between the ring and the caller's memory, where the page faults of a
 // fresh result spread over those threads.
-constexpr size_t kStageChunk = 4u << 20;   // bytes per chunk
+constexpr size_t kStageChunk = 4u << 20;   // bytes per chunk (2, 8 and 16 MiB measured no faster)
 constexpr int kStageSlots = 4;
 constexpr size_t kStageFrom = 4u << 20;    // smaller copies take the plain path (the ring's event waits cost more)
 
@@ -149,7 +174,7 @@ private:
         cpu_set_t set;
         int cores = 1;
         if (sched_getaffinity(0, sizeof(set), &set) == 0) cores = CPU_COUNT(&set);
-        int threads = std::min(cores, 8);
+        int threads = std::min(cores, 4);   // measured: eight threads are no faster on 25 MB and slower on 3 MB (wake-ups)
         if (const char* env = getenv("FTNN_HOST_COPY_THREADS")) threads = std::max(1, std::min(atoi(env), 16));   // tuning aid
         const int wanted = threads - 1;   // a caller pinned to one core (the reference's Makefile) copies alone
         // workers_ is final before the first worker runs: a slice's bounds depend on it
@@ -248,10 +273,81 @@ static void staged_download(void* host, const void* dev, size_t bytes) {
     }
 }
 
+// ---- copies below kStageFrom ----
+// Layer-sized tensors (a few MB) are where the reference's drivers spend their calls.  The runtime moves such
+// pageable memory at 118 us up and 195 us down for 3.2 MB, and takes 33 / 112 us for 64 / 256 KiB; the DMA engine on
+// pinned memory needs 65 us for the same 3.2 MB and 9 us for 64 KiB.  So these copies pass through pinned areas of
+// their own, one per kind of operand, each as large as the largest copy that takes this path: a chunk is copied
+// into (out of) the area while the DMA engine moves its neighbour.  An area is written again only by a later call,
+// and every host entry point returns after a download that has waited for the stream.
+constexpr size_t kSmallChunk = 1u << 20;
+constexpr size_t kSmallArea = kStageFrom;          // activations / rows, weights, results
+constexpr size_t kSmallThrArea = 256u << 10;       // thresholds: at most 65535 floats
+enum { AREA_ACT = 0, AREA_W, AREA_THR, AREA_DOWN, AREA_COUNT };
+
+struct SmallStage {
+    char* area[AREA_COUNT] = {};
+    hipEvent_t ev[kSmallArea / kSmallChunk] = {};
+};
+static SmallStage g_small;
+
+static SmallStage& small_stage() {
+    if (!g_small.area[0]) {
+        char* base = nullptr;
+        hip_or_die(hipHostMalloc((void**)&base, 3 * kSmallArea + kSmallThrArea, hipHostMallocDefault), "hipHostMalloc");
+        g_small.area[AREA_ACT] = base;
+        g_small.area[AREA_W] = base + kSmallArea;
+        g_small.area[AREA_DOWN] = base + 2 * kSmallArea;
+        g_small.area[AREA_THR] = base + 3 * kSmallArea;
+        for (hipEvent_t& e : g_small.ev) hip_or_die(hipEventCreateWithFlags(&e, hipEventDisableTiming), "hipEventCreate");
+    }
+    return g_small;
+}
+
+// host -> device through pinned area `area`; queued on the host stream, not waited for
+static void small_upload(void* dev, const void* host, size_t bytes, int area) {
+    char* pin = small_stage().area[area];
+    CopyPool& pool = CopyPool::get();
+    for (size_t off = 0; off < bytes; off += kSmallChunk) {
+        const size_t len = std::min(kSmallChunk, bytes - off);
+        pool.copy(pin + off, static_cast<const char*>(host) + off, len);
+        hip_or_die(hipMemcpyAsync(static_cast<char*>(dev) + off, pin + off, len, hipMemcpyHostToDevice, host_stream()), "H2D copy");
+    }
+}
+
+// device -> host after everything queued on the host stream; returns when `host` is complete
+static void small_download(void* host, const void* dev, size_t bytes) {
+    SmallStage& s = small_stage();
+    char* pin = s.area[AREA_DOWN];
+    CopyPool& pool = CopyPool::get();
+    hipStream_t st = host_stream();
+    int c = 0;
+    for (size_t off = 0; off < bytes; off += kSmallChunk, c++) {
+        const size_t len = std::min(kSmallChunk, bytes - off);
+        hip_or_die(hipMemcpyAsync(pin + off, static_cast<const char*>(dev) + off, len, hipMemcpyDeviceToHost, st), "D2H copy");
+        hip_or_die(hipEventRecord(s.ev[c], st), "hipEventRecord");
+    }
+    if (bytes == 0) hip_or_die(hipStreamSynchronize(st), "hipStreamSynchronize");
+    c = 0;
+    for (size_t off = 0; off < bytes; off += kSmallChunk, c++) {
+        const size_t len = std::min(kSmallChunk, bytes - off);
+        hip_or_die(hipEventSynchronize(s.ev[c]), "hipEventSynchronize");
+        pool.copy(static_cast<char*>(host) + off, pin + off, len);
+    }
+}
+
+static int area_of_slot(int slot);
+
 static void* upload(int slot, const void* host, size_t bytes) {
     void* d = dev_buf(slot, bytes);
-    if (bytes >= kStageFrom && CopyPool::get().parallel()) {
-        staged_upload(d, host, bytes);
+    const int area = area_of_slot(slot);
+    if (bytes >= kStageFrom) {
+        if (CopyPool::get().parallel()) {
+            staged_upload(d, host, bytes);
+            return d;
+        }
+    } else if (area >= 0 && bytes <= (area == AREA_THR ? kSmallThrArea : kSmallArea)) {
+        small_upload(d, host, bytes, area);
         return d;
     }
     hip_or_die(hipMemcpyAsync(d, host, bytes, hipMemcpyHostToDevice, host_stream()), "H2D copy");
@@ -259,8 +355,13 @@ static void* upload(int slot, const void* host, size_t bytes) {
 }
 
 static void download(void* host, const void* dev, size_t bytes) {
-    if (bytes >= kStageFrom && CopyPool::get().parallel()) {
-        staged_download(host, dev, bytes);
+    if (bytes >= kStageFrom) {
+        if (CopyPool::get().parallel()) {
+            staged_download(host, dev, bytes);
+            return;
+        }
+    } else {
+        small_download(host, dev, bytes);
         return;
     }
     hip_or_die(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, host_stream()), "D2H copy");
@@ -269,7 +370,20 @@ static void download(void* host, const void* dev, size_t bytes) {
 
 static void* host_alloc(size_t bytes, bool aligned32) {
     void* p;
-    if (aligned32) {
+    constexpr size_t kHuge = 2u << 20;
+    if (bytes >= kStageFrom) {
+        // A large result is often memory the process has not touched yet (a fresh mapping, or new heap), and the copy
+        // into it then pays a page fault per 4 KiB (25 MB: 2.6 ms on one thread, 1.1 ms on eight).  Its 2 MiB-aligned
+        // interior is therefore marked for transparent huge pages: 13 faults instead of 6300 (0.5 ms on one thread)
+        // where the memory is fresh, nothing where the allocator hands out memory that is mapped already.  Still
+        // plain heap memory that the caller free()s; where huge pages are unavailable the hint is ignored.
+        p = aligned32 ? aligned_alloc(32, (bytes + 31) / 32 * 32) : malloc(bytes);
+        if (p) {
+            const uintptr_t lo = (reinterpret_cast<uintptr_t>(p) + kHuge - 1) / kHuge * kHuge;
+            const uintptr_t hi = (reinterpret_cast<uintptr_t>(p) + bytes) / kHuge * kHuge;
+            if (hi > lo) (void)madvise(reinterpret_cast<void*>(lo), hi - lo, MADV_HUGEPAGE);
+        }
+    } else if (aligned32) {
         // aligned_alloc(32, ...) as src/tnns/ternarize2row_avx2.c:735
         p = aligned_alloc(32, (bytes + 31) / 32 * 32);
     } else {
@@ -283,6 +397,91 @@ static void* host_alloc(size_t bytes, bool aligned32) {
 }
 
 enum { SLOT_X = 0, SLOT_THR, SLOT_W, SLOT_ROWS, SLOT_SCRATCH, SLOT_Y };
+
+// the pinned area an operand below kStageFrom is staged through: the activation-side operand, the weight-side
+// operand and the thresholds of one call each have their own
+static int area_of_slot(int slot) {
+    switch (slot) {
+        case SLOT_X:
+        case SLOT_ROWS: return AREA_ACT;
+        case SLOT_W: return AREA_W;
+        case SLOT_THR: return AREA_THR;
+        default: return -1;
+    }
+}
+
+// ---- weights of tnns_conv, kept in engine form across calls ----
+// The reference's layer functions read the packed weights where they lie; here they must reach the device and, for
+// the matrix-core engine, be re-arranged into fragments: an upload, a launch and their latencies on every call for
+// data that a network never changes.  tnns_conv therefore keeps the prepared weights of the layers it has seen,
+// found again by host address, size, layer shape and a 64-bit hash of the CONTENTS, which is recomputed on every
+// call: a caller that frees the rows and packs another layer's at the same address, or rewrites them in place,
+// gets a different hash and a fresh upload.  Entries are dropped least recently used first beyond 512 entries or
+// 1 GiB of device memory.
+struct PreparedWeights {
+    const void* host;
+    size_t bytes;
+    uint64_t hash;
+    int type, C, KN, KH, KW;
+    void* dev;
+    size_t dev_bytes;
+    uint64_t last_use;
+};
+static std::vector<PreparedWeights> g_weights;
+static uint64_t g_weights_clock = 0;
+static size_t g_weights_bytes = 0;
+constexpr size_t kWeightCacheEntries = 512, kWeightCacheBytes = (size_t)1 << 30;
+
+// 64-bit hash of `bytes` (a multiple of 32: packed rows are whole groups of 4 words): four independent
+// multiply-rotate lanes over 32-byte blocks, folded at the end
+static uint64_t content_hash(const void* data, size_t bytes) {
+    const uint64_t* p = static_cast<const uint64_t*>(data);
+    uint64_t h0 = 0x9E3779B97F4A7C15ull, h1 = 0xC2B2AE3D27D4EB4Full, h2 = 0x165667B19E3779F9ull, h3 = 0x27D4EB2F165667C5ull;
+    auto rotl = [](uint64_t v, int r) { return (v << r) | (v >> (64 - r)); };
+    const size_t blocks = bytes / 32;
+    for (size_t i = 0; i < blocks; i++, p += 4) {
+        h0 = rotl((h0 ^ p[0]) * 0xFF51AFD7ED558CCDull, 29);
+        h1 = rotl((h1 ^ p[1]) * 0xC4CEB9FE1A85EC53ull, 31);
+        h2 = rotl((h2 ^ p[2]) * 0x9FB21C651E98DF25ull, 27);
+        h3 = rotl((h3 ^ p[3]) * 0xD6E8FEB86659FD93ull, 33);
+    }
+    const unsigned char* tail = reinterpret_cast<const unsigned char*>(p);
+    for (size_t i = 0; i < bytes % 32; i++) h0 = rotl((h0 ^ tail[i]) * 0xFF51AFD7ED558CCDull, 29);
+    uint64_t h = h0 ^ rotl(h1, 17) ^ rotl(h2, 34) ^ rotl(h3, 51) ^ (uint64_t)bytes;
+    h ^= h >> 33;
+    h *= 0xFF51AFD7ED558CCDull;
+    h ^= h >> 29;
+    return h;
+}
+
+// device pointer of the prepared weights of this layer (uploading and preparing them on a miss)
+static const void* prepared_weights(int type, const int64_t* host, size_t bytes, int C, int KN, int KH, int KW) {
+    const uint64_t hash = content_hash(host, bytes);
+    g_weights_clock++;
+    for (PreparedWeights& e : g_weights)
+        if (e.host == host && e.bytes == bytes && e.hash == hash && e.type == type && e.C == C && e.KN == KN && e.KH == KH &&
+            e.KW == KW) {
+            e.last_use = g_weights_clock;
+            return e.dev;
+        }
+    PreparedWeights e = {host, bytes, hash, type, C, KN, KH, KW, nullptr, (size_t)ftnn_conv_weights_bytes(type, C, KN, KH, KW),
+                         g_weights_clock};
+    while (!g_weights.empty() && (g_weights.size() >= kWeightCacheEntries || g_weights_bytes + e.dev_bytes > kWeightCacheBytes)) {
+        size_t oldest = 0;
+        for (size_t i = 1; i < g_weights.size(); i++)
+            if (g_weights[i].last_use < g_weights[oldest].last_use) oldest = i;
+        hip_or_die(hipStreamSynchronize(host_stream()), "hipStreamSynchronize");
+        hip_or_die(hipFree(g_weights[oldest].dev), "hipFree");
+        g_weights_bytes -= g_weights[oldest].dev_bytes;
+        g_weights.erase(g_weights.begin() + (long)oldest);
+    }
+    hip_or_die(hipMalloc(&e.dev, e.dev_bytes ? e.dev_bytes : 16), "hipMalloc");
+    int64_t* d_rows = (int64_t*)upload(SLOT_W, host, bytes);
+    if (ftnn_conv_prepare_weights(type, d_rows, C, KN, KH, KW, e.dev, host_stream()) != FTNN_OK) die("tnns_conv");
+    g_weights_bytes += e.dev_bytes;
+    g_weights.push_back(e);
+    return e.dev;
+}
 
 static int64_t* host_quantize_im2row(bool ternary, float* x, float* thr, int N, int C, int H, int W,
                                      int H_pad, int W_pad, int kH, int kW, int H_stride,
@@ -920,20 +1119,50 @@ void tnns_conv(testcase_t* t) {
         die("tnns_conv");
     const int w_tern = (type == kTNN || type == kBTN);
     const size_t rows = (size_t)N * OH * OW;
+    if (rows > 0x7fffffffull) {
+        fail(FTNN_EINVAL, "more than 2^31-1 output rows");
+        die("tnns_conv");
+    }
+    const size_t y_bytes = rows * KN * sizeof(float);
+    static const bool trace = getenv("FTNN_HOST_TRACE") != nullptr;   // tuning aid: phase times of every call on stderr
+    auto nowus = []() {
+        struct timespec ts;
+        clock_gettime(CLOCK_MONOTONIC, &ts);
+        return ts.tv_sec * 1e6 + ts.tv_nsec * 1e-3;
+    };
+    const double T0 = nowus();
+    float* y = (float*)host_alloc(y_bytes, false);   // before the device work: its pages can be mapped meanwhile
+    const double T1 = nowus();
     float* d_x = (float*)upload(SLOT_X, t->input, (size_t)N * C * H * W * sizeof(float));
     float* d_thr = (float*)upload(SLOT_THR, t->input_thresholds, (size_t)N * sizeof(float));
-    int64_t* d_w = (int64_t*)upload(SLOT_W, t->quantized_kernel_packing2,
-                                    (size_t)KN * ftnn_row_words(C, KH, KW, w_tern) * sizeof(int64_t));
+    const size_t w_bytes = (size_t)KN * ftnn_row_words(C, KH, KW, w_tern) * sizeof(int64_t);
     void* d_scr = dev_buf(SLOT_SCRATCH, (size_t)ftnn_conv_scratch_bytes(type, N, C, H, W, KN, KH, KW, t->paddingH,
                                                                   t->paddingW, t->strideH, t->strideW));
-    const size_t y_bytes = rows * KN * sizeof(float);
     float* d_y = (float*)dev_buf(SLOT_Y, y_bytes);
-    if (ftnn_conv(type, d_x, d_thr, d_w, N, C, H, W, KN, KH, KW, t->paddingH, t->paddingW,
-                  t->strideH, t->strideW, t->preluAlpha, d_scr, d_y,
-                  host_stream()) != FTNN_OK)
-        die("tnns_conv");
-    float* y = (float*)host_alloc(y_bytes, false);
+    const double T2 = nowus();
+    // a layer within the fp4 engine's 32-bit pixel indices (or on the vector ALU) takes its weights prepared
+    const bool prepared_ok =
+        select_conv_engine(type, N, C, H, W, KN, KH, KW, OH, OW) != FTNN_ENGINE_MFMA_F4 ||
+        ((int64_t)N * H * W * cpack_of(C) <= 0x7fffffffLL && (int64_t)rows * conv_f4_weight_words(C, KH, KW) <= 0x7fffffffLL);
+    int rc;
+    if (prepared_ok) {
+        const void* d_prep = prepared_weights(type, t->quantized_kernel_packing2, w_bytes, C, KN, KH, KW);
+        rc = ftnn_conv_prepared(type, d_x, d_thr, d_prep, N, C, H, W, KN, KH, KW, t->paddingH, t->paddingW, t->strideH,
+                                t->strideW, t->preluAlpha, d_scr, d_y, host_stream());
+    } else {
+        int64_t* d_w = (int64_t*)upload(SLOT_W, t->quantized_kernel_packing2, w_bytes);
+        rc = ftnn_conv(type, d_x, d_thr, d_w, N, C, H, W, KN, KH, KW, t->paddingH, t->paddingW, t->strideH, t->strideW,
+                       t->preluAlpha, d_scr, d_y, host_stream());
+    }
+    if (rc != FTNN_OK) die("tnns_conv");
+    const double T3 = nowus();
+    if (trace) hip_or_die(hipStreamSynchronize(host_stream()), "hipStreamSynchronize");   // separates kernels from download
+    const double T4 = nowus();
     download(y, d_y, y_bytes);
+    const double T5 = nowus();
+    if (trace)
+        fprintf(stderr, "tnns_conv: alloc %.0f, upload %.0f, weights + launch %.0f, kernels %.0f, download %.0f, total %.0f us\n",
+                T1 - T0, T2 - T1, T3 - T2, T4 - T3, T5 - T4, T5 - T0);
     t->output = y;  // src/tnns/tnns_cpu_mm_p2.c:119
 }
 

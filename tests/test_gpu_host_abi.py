@@ -132,3 +132,80 @@ def test_host_copies_with_other_thread_counts(threads):
     print("case host copy threads", threads, flush=True)
     r = subprocess.run([sys.executable, "-c", _CHILD, root], env=env, capture_output=True, text=True, timeout=110)
     assert r.returncode == 0 and "child ok" in r.stdout, r.stdout[-1500:] + r.stderr[-1500:]
+
+
+def _conv_at(hip, typ, L, qw_buf, alpha=0.5):
+    """tnns_conv with the packed weights at the address of qw_buf (no copy on the way in)"""
+    import ctypes as C
+    x, thr = np.ascontiguousarray(L["x"]), np.ascontiguousarray(L["thr"])
+    t = hip.Testcase(type=typ, batchcount=x.shape[0], channelcount=L["c"], inputW=L["iw"], inputH=L["ih"], kernelcount=L["kn"],
+                     kernelW=L["kw"], kernelH=L["kh"], paddingW=L["pad"], paddingH=L["pad"], strideW=L["stride"],
+                     strideH=L["stride"], preluAlpha=alpha, input_thresholds=thr.ctypes.data, input=x.ctypes.data,
+                     quantized_kernel_packing2=qw_buf.ctypes.data)
+    hip._L.tnns_conv(C.byref(t))
+    oh, ow = hip.out_dim(L["ih"], L["pad"], L["kh"], L["stride"]), hip.out_dim(L["iw"], L["pad"], L["kw"], L["stride"])
+    return hip._take(t.output, x.shape[0] * L["kn"] * oh * ow, np.float32)
+
+
+@pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
+def test_weights_rewritten_in_place_at_the_same_address(hip, oracle, typ):
+    """tnns_conv keeps a layer's weights on the device in engine form, found again by address, size and a hash of the
+    contents: rewriting the rows in place -- or packing another layer's into the same buffer, as the reference's
+    driver does when malloc hands the address out again (src/timing_layers.c:127-137,212-215) -- must be seen"""
+    wt = weight_is_ternary(typ)
+    shape = (128, 9, 9, 64, 3, 3, 1, 1)
+    L = make_layer(typ, shape, 2, seed=5100 + typ)
+    q1 = oracle.pack_weights(L["w"], L["wthr"], wt)
+    L2 = make_layer(typ, shape, 2, seed=5200 + typ)
+    q2 = oracle.pack_weights(L2["w"], L2["wthr"], wt)
+    assert q1.tobytes() != q2.tobytes()
+    buf = np.empty_like(q1)
+    for rep, q in enumerate((q1, q1, q2, q2, q1)):
+        buf[:] = q                                  # same address every time
+        want = oracle.conv(typ, L["x"], L["thr"], q, L["kn"], 3, 3, 1, 1, 0.5).reshape(-1)
+        got = _conv_at(hip, typ, L, buf)
+        assert got.tobytes() == want.tobytes(), rep
+    # one flipped lane is another layer too
+    buf[:] = q1
+    buf[3] ^= 1 << 17
+    want = oracle.conv(typ, L["x"], L["thr"], buf.copy(), L["kn"], 3, 3, 1, 1, 0.5).reshape(-1)
+    assert _conv_at(hip, typ, L, buf).tobytes() == want.tobytes()
+    # the same address and bytes under another layer shape (same row length, other kernel count / channel split)
+    shape_b = (64, 9, 9, 128, 3, 3, 1, 1)
+    Lb = make_layer(typ, shape_b, 2, seed=5300 + typ)
+    qb = oracle.pack_weights(Lb["w"], Lb["wthr"], wt)
+    if qb.size == buf.size:
+        buf[:] = qb
+        want = oracle.conv(typ, Lb["x"], Lb["thr"], qb, Lb["kn"], 3, 3, 1, 1, 0.5).reshape(-1)
+        assert _conv_at(hip, typ, Lb, buf).tobytes() == want.tobytes()
+
+
+def test_more_layers_than_the_weight_cache_holds(hip, oracle):
+    """600 distinct small layers, then the first ones again: entries are dropped least recently used first and come back"""
+    L = make_layer(TNN, (64, 5, 5, 32, 3, 3, 1, 1), 1, seed=6000)
+    rng = np.random.default_rng(6)
+    packs, wants = [], []
+    for i in range(600):
+        w = rng.integers(-1, 2, size=(32, 64, 3, 3)).astype(np.float32)
+        q = oracle.pack_weights(w, np.full(32, 0.5, np.float32), True)
+        packs.append(q)
+        if i < 3 or i > 596:
+            wants.append((i, oracle.conv(TNN, L["x"], L["thr"], q, 32, 3, 3, 1, 1, 0.5).reshape(-1)))
+        got = _conv_at(hip, TNN, L, q)
+        if i < 3 or i > 596:
+            assert got.tobytes() == wants[-1][1].tobytes(), i
+    for i, want in wants:
+        assert _conv_at(hip, TNN, L, packs[i]).tobytes() == want.tobytes(), i
+
+
+@pytest.mark.parametrize("pixels", [127, 512, 1023, 1024, 1025, 4095])
+def test_copy_sizes_around_the_staging_chunks(hip, oracle, pixels):
+    """tensors from half a KiB to just under 4 MiB go through the small pinned areas in chunks of 1 MiB: sizes below,
+    at and above whole chunks, results up to 4 MiB minus a row"""
+    c, kn = 64, 250                                    # x: pixels * 256 B, y: pixels * 1000 B
+    L = make_layer(TBN, (c, 1, pixels, kn, 1, 1, 0, 1), 1, seed=6400 + pixels)
+    qw = oracle.pack_weights(L["w"], L["wthr"], False)
+    want = oracle.conv(TBN, L["x"], L["thr"], qw, kn, 1, 1, 0, 1, 0.5)
+    for rep in range(2):
+        got = hip.host_conv(TBN, L["x"], L["thr"], qw, kn, 1, 1, 0, 1, 0.5)
+        assert got.tobytes() == want.tobytes(), rep
