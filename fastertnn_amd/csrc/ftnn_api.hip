@@ -41,6 +41,16 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // words per operand row (one plane) that every engine's 32-bit sums and offsets hold
 constexpr int kMaxRowWords = (1 << 24) - 4;
 
+// whether rows of ceil(C/64) * KH * KW words are within what 32-bit sums and offsets hold; no intermediate product
+// overflows whatever the (positive) arguments are
+static bool row_fits(int C, int KH, int KW) {
+    int64_t k;
+    if (C > (1 << 30) || __builtin_mul_overflow((int64_t)KH, (int64_t)KW, &k) ||
+        __builtin_mul_overflow(k, ((int64_t)C + 63) / 64, &k))
+        return false;
+    return k <= kMaxRowWords;
+}
+
 // common conv-shape validation; fills OH/OW
 int check_conv_shape(int N, int C, int H, int W, int H_pad, int W_pad, int kH, int kW,
                             int H_stride, int W_stride, int* OH, int* OW) {
@@ -56,7 +66,7 @@ int check_conv_shape(int N, int C, int H, int W, int H_pad, int W_pad, int kH, i
     if (Hp > 0x3ffffffLL || Wp > 0x3ffffffLL || Hp * Wp > 0x3ffffffLL)
         return fail(FTNN_EINVAL, "padded image plane above the supported 2^26 pixels");
     // 32-bit accumulators count up to 128 per word of a row
-    if (C > (1 << 30) || ((int64_t)C + 63) / 64 * kH * kW > kMaxRowWords)
+    if (!row_fits(C, kH, kW))
         return fail(FTNN_EINVAL, "more than %d words per im2row row", kMaxRowWords);
     *OH = out_dim(H, H_pad, kH, H_stride);
     *OW = out_dim(W, W_pad, kW, W_stride);
@@ -723,14 +733,20 @@ int ftnn_out_dim(int in, int pad, int k, int stride) { return out_dim(in, pad, k
 
 int64_t ftnn_row_words(int C, int KH, int KW, int ternary) {
     if (C <= 0 || KH <= 0 || KW <= 0) return 0;
-    const int64_t k = ((int64_t)C + 63) / 64 * KH * KW;
+    int64_t k;   // the window alone can exceed 64 bits: KH * KW up to 2^62 times 2^25 channel words
+    if (__builtin_mul_overflow((int64_t)KH, (int64_t)KW, &k) || __builtin_mul_overflow(k, ((int64_t)C + 63) / 64, &k)) return 0;
     if (k > kMaxRowWords) return 0;
     const int64_t kw = (k + 3) / 4 * 4;
     return ternary ? 2 * kw : kw;
 }
 
 int64_t ftnn_pack_scratch_bytes(int N, int C, int H, int W, int ternary) {
-    return (int64_t)N * H * W * cpack_of(C) * (ternary ? 16 : 8);
+    if (N <= 0 || C <= 0 || H <= 0 || W <= 0) return 0;
+    int64_t bytes;   // 0 for a tensor whose packed copy does not fit 63 bits (no such tensor passes the shape checks)
+    if (__builtin_mul_overflow((int64_t)N * cpack_of(C), (int64_t)H * W, &bytes) ||
+        __builtin_mul_overflow(bytes, (int64_t)(ternary ? 16 : 8), &bytes))
+        return 0;
+    return bytes;
 }
 
 // Layer engine by shape, from measurements on MI355X: the fp4 matrix-core kernel wins wherever it
@@ -968,7 +984,7 @@ static int64_t prepared_bytes(int type, int C, int KN, int KH, int KW, int64_t* 
 
 int64_t ftnn_conv_weights_bytes(int type, int C, int KN, int KH, int KW) {
     if (type < kTNN || type > kBNN || C <= 0 || KN <= 0 || KH <= 0 || KW <= 0) return 0;
-    if (C > (1 << 30) || ((int64_t)C + 63) / 64 * KH * KW > kMaxRowWords) return 0;
+    if (!row_fits(C, KH, KW)) return 0;
     return prepared_bytes(type, C, KN, KH, KW, nullptr);
 }
 
@@ -976,7 +992,7 @@ int ftnn_conv_prepare_weights(int type, const int64_t* d_qw, int C, int KN, int 
                               void* stream) {
     if (type < kTNN || type > kBNN) return fail(FTNN_EINVAL, "unknown network type %d", type);
     if (C <= 0 || KN <= 0 || KH <= 0 || KW <= 0) return fail(FTNN_EINVAL, "non-positive dimension");
-    if (C > (1 << 30) || ((int64_t)C + 63) / 64 * KH * KW > kMaxRowWords)
+    if (!row_fits(C, KH, KW))
         return fail(FTNN_EINVAL, "more than %d words per weight row", kMaxRowWords);
     if (!d_qw || !d_prepared || !aligned16(d_qw) || !aligned16(d_prepared))
         return fail(FTNN_EINVAL, "null or misaligned device pointer");
@@ -1058,7 +1074,7 @@ int ftnn_conv_static(int type, const float* d_x, const float* d_thr, const int64
 int ftnn_pack_weights(int ternary, const float* d_w, const float* d_thr, int KN, int C, int KH,
                       int KW, int64_t* d_out, void* stream) {
     if (KN <= 0 || C <= 0 || KH <= 0 || KW <= 0) return fail(FTNN_EINVAL, "non-positive dimension");
-    if (C > (1 << 30) || ((int64_t)C + 63) / 64 * KH * KW > kMaxRowWords)
+    if (!row_fits(C, KH, KW))
         return fail(FTNN_EINVAL, "more than %d words per weight row", kMaxRowWords);
     if (!d_w || !d_thr || !d_out) return fail(FTNN_EINVAL, "null device pointer");
     hipError_t e = launch_pack_weights(ternary != 0, d_w, d_thr, KN, C, KH, KW, d_out,

@@ -7,7 +7,7 @@ namespace ftnn {
 
 constexpr int kTNN = 0, kTBN = 1, kBTN = 2, kBNN = 3;
 
-inline int cpack_of(int C) { return (C + 63) / 64; }
+inline int cpack_of(int C) { return (int)(((int64_t)C + 63) / 64); }
 inline int round4(int k) { return 4 * ((k + 3) / 4); }
 inline int out_dim(int in, int pad, int k, int stride) { return (in + 2 * pad - k) / stride + 1; }
 
