@@ -49,11 +49,10 @@ print("child ok")
 """
 
 
-@pytest.mark.parametrize("split", ["auto", "1", "2", "4"])
-@pytest.mark.parametrize("buffer_loads", ["off", "on"])
+# ("on", "auto") is the default configuration, which every other suite covers
+@pytest.mark.parametrize("buffer_loads,split", [("off", "auto"), ("off", "1"), ("off", "2"), ("off", "4"), ("on", "1"), ("on", "2"),
+                                                ("on", "4")])
 def test_layer_kernel_variants(split, buffer_loads):
-    if split == "auto" and buffer_loads == "on":
-        pytest.skip("the default configuration: covered by every other suite")
     env = dict(os.environ)
     if buffer_loads == "off":
         env["FTNN_CONV_NO_BUFFER_LOADS"] = "1"
