@@ -17,7 +17,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hi
 # that the compiler keeps in scratch memory could be the target of a load in flight, and every scratch access is
 # itself a vector-memory operation that moves the count the waits rely on.  The build refuses scratch use in
 # them (the library checks the same at run time before the first launch).  Source -> name fragments.
-NO_SCRATCH = {"mfma_kernels.hip": ("k_conv_f4", "k_mfma")}
+NO_SCRATCH = {"mfma_kernels.hip": ("k_conv_f4", "k_mfma")}   # "k_mfma" covers k_mfma_p4 as well
 
 
 def check_no_scratch(src, remarks):

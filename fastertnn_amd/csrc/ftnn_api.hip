@@ -845,8 +845,8 @@ int64_t ftnn_mm_scratch_bytes(int engine, int type, int N, int OH, int OW, int K
     const int Kw = round4(K);
     if (engine == FTNN_ENGINE_AUTO) engine = select_engine(type, M, KN, Kw);
     if (engine != FTNN_ENGINE_MFMA_I8 && engine != FTNN_ENGINE_MFMA_F4) return 0;
-    const bool f4 = engine == FTNN_ENGINE_MFMA_F4;
-    return mfma_fragment_bytes(f4, M, Kw) + mfma_fragment_bytes(f4, KN, Kw);
+    if (engine == FTNN_ENGINE_MFMA_F4) return mfma_packed4_bytes(M, Kw) + mfma_packed4_bytes(KN, Kw);
+    return mfma_fragment_bytes(false, M, Kw) + mfma_fragment_bytes(false, KN, Kw);
 }
 
 static int check_mfma_engine(int engine, int Kw) {
@@ -859,7 +859,7 @@ static int check_mfma_engine(int engine, int Kw) {
 
 int64_t ftnn_expand_bytes(int engine, int rows, int K) {
     if (rows <= 0 || K <= 0 || K > kMaxRowWords || (engine != FTNN_ENGINE_MFMA_I8 && engine != FTNN_ENGINE_MFMA_F4)) return 0;
-    return mfma_fragment_bytes(engine == FTNN_ENGINE_MFMA_F4, rows, round4(K));
+    return engine == FTNN_ENGINE_MFMA_F4 ? mfma_packed4_bytes(rows, round4(K)) : mfma_fragment_bytes(false, rows, round4(K));
 }
 
 int ftnn_expand_rows(int engine, int ternary, const int64_t* d_rows, int rows, int K, void* d_out,
@@ -869,8 +869,9 @@ int ftnn_expand_rows(int engine, int ternary, const int64_t* d_rows, int rows, i
     if (rc != FTNN_OK) return rc;
     if (!d_rows || !d_out || !aligned16(d_rows) || !aligned16(d_out))
         return fail(FTNN_EINVAL, "null or misaligned device pointer");
-    hipError_t e = launch_mfma_expand(engine == FTNN_ENGINE_MFMA_F4, ternary != 0, d_rows, rows, round4(K),
-                                      d_out, (hipStream_t)stream);
+    hipError_t e = engine == FTNN_ENGINE_MFMA_F4
+                       ? launch_mfma_pack4(ternary != 0, d_rows, rows, round4(K), d_out, (hipStream_t)stream)
+                       : launch_mfma_expand(false, ternary != 0, d_rows, rows, round4(K), d_out, (hipStream_t)stream);
     return e == hipSuccess ? FTNN_OK : hip_fail(e, "expand launch");
 }
 
@@ -886,8 +887,11 @@ int ftnn_mm_expanded(int engine, int type, const void* d_a_exp, const void* d_b_
     if (M > 0x7fffffffLL) return fail(FTNN_EINVAL, "more than 2^31-1 output rows");
     if (!d_a_exp || !d_b_exp || !d_y || !aligned16(d_a_exp) || !aligned16(d_b_exp))
         return fail(FTNN_EINVAL, "null or misaligned device pointer");
-    hipError_t e = launch_mfma_gemm(engine == FTNN_ENGINE_MFMA_F4, type, d_a_exp, d_b_exp, M, OH * OW, KN,
-                                    round4(K), K_unpack, prelu_alpha, d_y, (hipStream_t)stream);
+    hipError_t e = engine == FTNN_ENGINE_MFMA_F4
+                       ? launch_mfma_gemm_packed4(type, d_a_exp, d_b_exp, M, OH * OW, KN, round4(K), K_unpack, prelu_alpha, d_y,
+                                                  (hipStream_t)stream)
+                       : launch_mfma_gemm(false, type, d_a_exp, d_b_exp, M, OH * OW, KN, round4(K), K_unpack, prelu_alpha, d_y,
+                                          (hipStream_t)stream);
     return e == hipSuccess ? FTNN_OK : hip_fail(e, "mfma gemm launch");
 }
 

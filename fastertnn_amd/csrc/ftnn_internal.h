@@ -254,6 +254,12 @@ hipError_t launch_mfma_expand(bool f4, bool ternary, const int64_t* d_rows, int 
                               hipStream_t st);
 hipError_t launch_mfma_gemm(bool f4, int type, const void* d_af, const void* d_bf, int64_t M, int OHW, int KN,
                             int Kw, int K_unpack, float alpha, float* d_y, hipStream_t st);
+// the fp4 GEMM's own operand form, two bits per lane ("packed4"): what ftnn_expand_rows / ftnn_mm_expanded /
+// ftnn_mm_engine use for FTNN_ENGINE_MFMA_F4 (the layer kernels keep the plain fragments above)
+int64_t mfma_packed4_bytes(int64_t rows, int Kw);
+hipError_t launch_mfma_pack4(bool ternary, const int64_t* d_rows, int rows, int Kw, void* d_out, hipStream_t st);
+hipError_t launch_mfma_gemm_packed4(int type, const void* d_ac, const void* d_bc, int64_t M, int OHW, int KN, int Kw, int K_unpack,
+                                    float alpha, float* d_y, hipStream_t st);
 hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* d_b, int64_t M, int OHW,
                           int KN, int Kw, int K_unpack, float alpha, float* d_y, void* d_scratch,
                           hipStream_t st);

@@ -168,6 +168,42 @@ __device__ __forceinline__ void dma16(const uint4* gsrc, uint32_t lds_byte_addr)
                  : "memory");
 }
 
+// Epilogue of the GEMM kernels: r = acc - bias, then PReLU in the reference's form for the type (form 0 "f = r; if
+// (f <= 0) f *= alpha", mm_p2_final_tnn_avx2.c:204-208; form 1 "r >= 0 ? r : alpha * r", mm_p2_final_tbn_avx2.c:73), stored
+// row-major (SWAP = false, OHW == 1) or in NCHW order.  Accumulator e of block (a, b): P row = 32 * (prb + a) + 8 * (e / 4)
+// + 4 * (lane / 32) + e % 4, Q row = 32 * (qrb + b) + lane % 32.
+template <bool F4, bool SWAP, int WT>
+__device__ __forceinline__ void store_tile(const typename Acc<F4>::type (&acc)[WT][WT], float* __restrict__ Y, int M, int KN,
+                                           int OHW, int prb, int qrb, int lane, int bias, int form, float alpha) {
+    const bool le_form = form == 0;
+#pragma unroll
+    for (int a = 0; a < WT; a++)
+#pragma unroll
+        for (int b = 0; b < WT; b++) {
+            const int q = (qrb + b) * 32 + (lane & 31);
+            const int pbase = (prb + a) * 32 + 4 * (lane >> 5);
+            size_t qoff;
+            if (SWAP) {   // q = i is fixed per block: split it into (image, pixel) once
+                const int img = q / OHW;
+                qoff = (size_t)img * KN * OHW + (q - img * OHW);
+            } else {
+                qoff = (size_t)q;
+            }
+            const bool qok = q < (SWAP ? M : KN);
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int p = pbase + 8 * (e >> 2) + (e & 3);
+                const int r = (int)acc[a][b][e] - bias;
+                const float fr = (float)r;
+                // form 0: scale when f <= 0 (a zero becomes 0 * alpha); form 1: scale when r < 0
+                const bool scale = le_form ? (fr <= 0.0f) : (r < 0);
+                const float f = scale ? fr * alpha : fr;
+                const size_t o = SWAP ? qoff + (size_t)p * OHW : (size_t)p * KN + qoff;
+                if (qok && p < (SWAP ? KN : M)) Y[o] = f;
+            }
+        }
+}
+
 // P operand = MFMA A side (its rows index the accumulator registers), Q operand = MFMA B
 // side (its rows run along the lanes).  SWAP = false: P = activation rows i, Q = weight
 // rows j (lanes along j: contiguous for a row-major m x n result).  SWAP = true: P =
@@ -282,35 +318,200 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
     for (; s + kNS < nstep; s++) step_body(s, std::true_type{});
     for (; s < nstep; s++) step_body(s, std::false_type{});
 
-    // accumulator e of block (a, b): P row = 32*prb + 8*(e/4) + 4*(lane/32) + e%4, Q row = 32*qrb + lane%32.
-    // SWAP = false is only launched for OHW == 1 (row-major m x n result).
-    const bool le_form = form == 0;
+    store_tile<F4, SWAP, WT>(acc, Y, M, KN, OHW, prb0 + wy * WT, qrb0 + wx * WT, lane, bias, form, alpha);
+}
+
+// ------------------------------------------------- fp4 operands at two bits per lane
+// The fp4 GEMM above is bound by what it moves, not by its schedule: the stream of operand fragments from L2 into LDS
+// (8 GiB per 8192 x 8192 x 32768 launch) holds the chip's clock down.  A ternary or binary lane carries two bits of
+// information, and an E2M1 nibble of -1 / 0 / +1 uses two of its four bits: 0x2 | sign << 3, i.e. bits 1 and 3 (a
+// zero lane may keep its sign bit: -0 multiplies like +0).  Two dwords of nibbles D0, D1 therefore share one dword,
+// P = D0 | D1 >> 1, and come apart again with D0 = P & 0xAAAAAAAA, D1 = (P << 1) & 0xAAAAAAAA: 1.5 vector instructions
+// per dword, which the wavefronts issue beside their MFMAs.  Operands in this form ("packed4") are half the bytes in HBM,
+// through L2 -> LDS and through the LDS reads.
+//
+// Layout: 1 KiB blocks [row block of 32][pair of K words][lane l = (k half l / 32, row l % 32)][16 bytes], the 16 bytes of a
+// lane being (P0, P1) of the even K word and (P0, P1) of the odd one, P0 = D0 | D1 >> 1, P1 = D2 | D3 >> 1 with D0..D3 the
+// lane's 16 bytes of the plain fragment layout above.  One LDS-direct load of 16 bytes per lane moves a row block's two
+// K words, so a step of two K words takes half the load and half the LDS-read instructions of the plain kernel as well.
+
+// grid (row blocks, groups / 4), block 256: as k_expand<true, TERN>, writing the packed4 layout (Kw words per row)
+template <bool TERN>
+__global__ __launch_bounds__(256) void k_pack4(const uint32_t* __restrict__ P, int rows, int G, uint2* __restrict__ out) {
+    constexpr int kGPB = 4;
+    constexpr int DPG = TERN ? 16 : 8;        // dwords per group and row
+    constexpr int RD = kGPB * DPG;            // dwords per row in the block
+    constexpr int RS = RD + 1;                // LDS row stride: odd, the 32 rows of a read hit 32 banks
+    __shared__ uint32_t stage[32 * RS];
+    const int rb = blockIdx.x, g0 = blockIdx.y * kGPB, t = threadIdx.x;
+    {
+        constexpr int PPR = RD / 4;           // 16-byte pieces per row
+        const int gmax = min(kGPB, G - g0) * (DPG / 4);
+#pragma unroll
+        for (int k = 0; k < (32 * PPR) / 256; k++) {
+            const int idx = t + 256 * k, rr = idx / PPR, pc = idx - rr * PPR;
+            const int srow = min(rb * 32 + rr, rows - 1);
+            uint4 v = make_uint4(0u, 0u, 0u, 0u);
+            if (pc < gmax) v = *reinterpret_cast<const uint4*>(P + ((size_t)srow * G + g0) * DPG + pc * 4);
+            uint32_t* d = stage + rr * RS + pc * 4;
+            d[0] = v.x;
+            d[1] = v.y;
+            d[2] = v.z;
+            d[3] = v.w;
+        }
+    }
+    __syncthreads();
+    const int r = t & 31, dq = t >> 5;        // dq: dword of the group = (K word dq / 2, k half dq % 2)
+    const bool live = rb * 32 + r < rows;
+#pragma unroll
+    for (int i = 0; i < kGPB; i++) {
+        const int g = g0 + i;
+        if (g >= G) break;
+        const uint32_t sv = stage[r * RS + i * DPG + dq];
+        const uint32_t zv = TERN ? stage[r * RS + i * DPG + 8 + dq] : 0u;
+        const uint32_t nz = live ? ~zv : 0u;
+        const uint32_t s = sv & nz;
+        uint32_t o[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {   // 8 lanes -> 8 nibbles: bit i lands on bit 4 i
+            uint32_t a = (s >> (8 * q)) & 0xffu, b = (nz >> (8 * q)) & 0xffu;
+            a = (a | (a << 12)) & 0x000F000Fu;
+            a = (a | (a << 6)) & 0x03030303u;
+            a = (a | (a << 3)) & 0x11111111u;
+            b = (b | (b << 12)) & 0x000F000Fu;
+            b = (b | (b << 6)) & 0x03030303u;
+            b = (b | (b << 3)) & 0x11111111u;
+            o[q] = (a << 3) | (b << 1);
+        }
+        const int w = g * 4 + (dq >> 1), h = dq & 1;   // K word and k half of this thread's 32 lanes
+        const size_t block = (size_t)rb * (G * 2) + (w >> 1);
+        out[(block * 64 + h * 32 + r) * 2 + (w & 1)] = make_uint2(o[0] | (o[1] >> 1), o[2] | (o[3] >> 1));
+    }
+}
+
+// (P0, P1) of one K word -> the lane's 16 bytes of nibbles
+__device__ __forceinline__ uint4 unpack4(uint32_t p0, uint32_t p1) {
+    constexpr uint32_t m = 0xAAAAAAAAu;
+    return make_uint4(p0 & m, (p0 << 1) & m, p1 & m, (p1 << 1) & m);
+}
+
+// The fp4 GEMM on packed4 operands.  Same tiling as k_mfma<true, ...> (2 x 2 wavefronts, WT x WT blocks of 32 x 32 each,
+// steps of two K words, ring of kNS stages filled by LDS-direct loads that the kernel counts by hand), with one 1 KiB block
+// per row block and step.  A step: the first K word's 16 multiplies run while the second one's operands are unpacked;
+// then the barrier; the second K word's multiplies run beside the loads of stage s + kNS, the LDS reads of stage s + 1
+// and the unpacking of its first K word.
+template <bool SWAP, int WT, int kNS>
+__global__ __launch_bounds__(256) void k_mfma_p4(const uint4* __restrict__ Pc, const uint4* __restrict__ Qc, float* __restrict__ Y,
+                                                 int M, int KN, int OHW, int KP, int bias, int form, float alpha) {
+    extern __shared__ uint4 lds[];   // kNS stages of kFR KiB
+    typedef typename Acc<true>::type acc_t;
+    constexpr int RB = 2 * WT, kFR = 2 * RB, kFW = kFR / 4, NL = 2 * WT;   // kFW = WT blocks staged per wavefront and step
+    static_assert(NL % kFW == 0 && (NL / 2) % 2 == 0, "loads and reads spread evenly over the slots");
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wy = wave >> 1, wx = wave & 1;
+    const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN;
+    const int prb0 = blockIdx.x * RB, qrb0 = blockIdx.y * RB;
+    const int prbmax = (prow + 31) / 32 - 1, qrbmax = (qrow + 31) / 32 - 1;
+    acc_t acc[WT][WT];
 #pragma unroll
     for (int a = 0; a < WT; a++)
 #pragma unroll
-        for (int b = 0; b < WT; b++) {
-            const int q = (qrb0 + wx * WT + b) * 32 + (lane & 31);
-            const int pbase = (prb0 + wy * WT + a) * 32 + 4 * (lane >> 5);
-            size_t qoff;
-            if (SWAP) {   // q = i is fixed per block: split it into (image, pixel) once
-                const int img = q / OHW;
-                qoff = (size_t)img * KN * OHW + (q - img * OHW);
-            } else {
-                qoff = (size_t)q;
-            }
-            const bool qok = q < (SWAP ? M : KN);
+        for (int b = 0; b < WT; b++)
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int p = pbase + 8 * (e >> 2) + (e & 3);
-                const int r = (int)acc[a][b][e] - bias;
-                const float fr = (float)r;
-                // form 0: scale when f <= 0 (a zero becomes 0 * alpha); form 1: scale when r < 0
-                const bool scale = le_form ? (fr <= 0.0f) : (r < 0);
-                const float f = scale ? fr * alpha : fr;
-                const size_t o = SWAP ? qoff + (size_t)p * OHW : (size_t)p * KN + qoff;
-                if (qok && p < (SWAP ? KN : M)) Y[o] = f;
-            }
+            for (int e = 0; e < 16; e++) acc[a][b][e] = 0;
+
+    // block f of a stage: side f / RB (0 = P, 1 = Q), row block f % RB; row blocks past the operand are clamped
+    const uint4* src[kFW];
+#pragma unroll
+    for (int i = 0; i < kFW; i++) {
+        const int f = wave * kFW + i;
+        const int side = f / RB, rbi = f % RB;
+        const uint4* base = side == 0 ? Pc + (size_t)min(prb0 + rbi, prbmax) * KP * 64 : Qc + (size_t)min(qrb0 + rbi, qrbmax) * KP * 64;
+        src[i] = base + lane;
+    }
+    const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)lds);
+    const int nstep = KP;
+    auto stage = [&](int step) {
+        const uint32_t dst = lds0 + (uint32_t)(step % kNS) * (kFR * 1024) + wave * (kFW * 1024);
+#pragma unroll
+        for (int i = 0; i < kFW; i++) dma16(src[i] + (size_t)step * 64, dst + i * 1024);
+    };
+    // raw: the packed blocks of the stage being consumed; e[k]: the unpacked operands of its K word k.  Slots in the
+    // order the multiplies take them: 0: P block 0, 1..WT: Q blocks, then P blocks 1..WT-1.
+    uint4 ra[WT], rq[WT], ea[2][WT], eq[2][WT];
+    auto read_raw = [&](int buf, int i) {
+        const uint4* L = lds + (size_t)buf * kFR * 64;
+        if (i == 0) ra[0] = L[(wy * WT + 0) * 64 + lane];
+        else if (i <= WT) rq[i - 1] = L[(RB + wx * WT + (i - 1)) * 64 + lane];
+        else ra[i - WT] = L[(wy * WT + (i - WT)) * 64 + lane];
+    };
+    auto unpack = [&](int k, int i) {
+        const uint4& r = i == 0 ? ra[0] : (i <= WT ? rq[i - 1] : ra[i - WT]);
+        const uint4 v = k == 0 ? unpack4(r.x, r.y) : unpack4(r.z, r.w);
+        if (i == 0) ea[k][0] = v;
+        else if (i <= WT) eq[k][i - 1] = v;
+        else ea[k][i - WT] = v;
+    };
+    auto mfma2 = [&](int k, int i) {
+#pragma unroll
+        for (int j = 0; j < WT / 2; j++) {
+            const int m = (WT / 2) * i + j;
+            mfma<true>(acc[m / WT][m % WT], ea[k][m / WT], eq[k][m % WT]);
         }
+    };
+
+    // prologue: the first kNS stages in flight, wait for stage 0 only
+#pragma unroll
+    for (int p = 0; p < kNS; p++)
+        if (p < nstep) stage(p);
+    if (nstep >= kNS) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFW * (kNS - 1)) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NL; i++) read_raw(0, i);
+#pragma unroll
+    for (int i = 0; i < NL; i++) unpack(0, i);
+
+    auto step_body = [&](int s, auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;   // FULL: s + kNS < nstep
+        // first K word: multiply, and unpack the second one's operands (their packed blocks arrived a phase ago)
+#pragma unroll
+        for (int i = 0; i < NL; i++) {
+            unpack(1, i);
+            mfma2(0, i);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // Everything of this stage is in registers.  Stage s + 1 must have landed (stages s + 2 .. s + kNS - 1 may
+        // still be in flight); after the barrier buffer s % kNS is free for stage s + kNS.
+        if (FULL || s + kNS - 1 < nstep) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFW * (kNS - 2)) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        const bool do_ld = FULL || s + 1 < nstep;
+        const uint32_t dst = lds0 + (uint32_t)(s % kNS) * (kFR * 1024) + wave * (kFW * 1024);
+        // second K word: first half of the slots issue the LDS reads of the next stage (two per slot) and its loads,
+        // the second half unpacks the next stage's first K word (two blocks per slot)
+#pragma unroll
+        for (int i = 0; i < NL; i++) {
+            if (i < NL / 2) {
+                if (do_ld) {
+                    read_raw((s + 1) % kNS, 2 * i);
+                    read_raw((s + 1) % kNS, 2 * i + 1);
+                }
+                if (FULL && i < kFW) dma16(src[i] + (size_t)(s + kNS) * 64, dst + i * 1024);
+            } else if (do_ld) {
+                unpack(0, 2 * (i - NL / 2));
+                unpack(0, 2 * (i - NL / 2) + 1);
+            }
+            mfma2(1, i);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    int s = 0;
+    for (; s + kNS < nstep; s++) step_body(s, std::true_type{});
+    for (; s < nstep; s++) step_body(s, std::false_type{});
+
+    store_tile<true, SWAP, WT>(acc, Y, M, KN, OHW, prb0 + wy * WT, qrb0 + wx * WT, lane, bias, form, alpha);
 }
 
 // ------------------------------------------------------------ conv layer (fp4)
@@ -801,6 +1002,36 @@ hipError_t launch_expand(bool tern, const uint32_t* rows_ptr, int rows, int G, u
     return hipGetLastError();
 }
 
+template <bool SWAP, int WT, int NS>
+hipError_t launch_gemm_p4_tile(const uint4* Pc, const uint4* Qc, float* Y, int M, int KN, int OHW, int KP, int bias, int form,
+                               float alpha, hipStream_t st) {
+    auto kern = k_mfma_p4<SWAP, WT, NS>;
+    constexpr size_t lds_bytes = (size_t)NS * 4 * WT * 1024;
+    // hand-counted LDS-direct loads: no scratch (see launch_gemm_tile); the opt-in to more than 64 KiB of LDS is per kernel
+    static const hipError_t configured = []() {
+        const void* k = reinterpret_cast<const void*>(&k_mfma_p4<SWAP, WT, NS>);
+        hipFuncAttributes attr;
+        hipError_t e = hipFuncGetAttributes(&attr, k);
+        if (e == hipSuccess && attr.localSizeBytes != 0) e = hipErrorLaunchFailure;
+        if (e != hipSuccess) return e;
+        return hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)NS * 4 * WT * 1024));
+    }();
+    if (configured != hipSuccess) return configured;
+    const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN, edge = 64 * WT;
+    dim3 grid((prow + edge - 1) / edge, (qrow + edge - 1) / edge);
+    if (grid.y > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, st, Pc, Qc, Y, M, KN, OHW, KP, bias, form, alpha);
+    return hipGetLastError();
+}
+
+template <bool SWAP>
+hipError_t launch_gemm_p4(const uint4* Pc, const uint4* Qc, float* Y, int M, int KN, int OHW, int KP, int bias, int form,
+                          float alpha, hipStream_t st) {
+    const int64_t big = (((int64_t)M + 255) / 256) * ((KN + 255) / 256);
+    return big < mfma_small_tile_below() ? launch_gemm_p4_tile<SWAP, 2, 4>(Pc, Qc, Y, M, KN, OHW, KP, bias, form, alpha, st)
+                                         : launch_gemm_p4_tile<SWAP, 4, 4>(Pc, Qc, Y, M, KN, OHW, KP, bias, form, alpha, st);
+}
+
 }  // namespace
 
 int64_t mfma_fragment_bytes(bool f4, int64_t rows, int Kw) {
@@ -832,6 +1063,28 @@ hipError_t launch_mfma_gemm(bool f4, int type, const void* d_af, const void* d_b
     }
     return swap ? launch_gemm<false, true>(Bf, Af, d_y, (int)M, KN, OHW, KB, bias, form, alpha, st)
                 : launch_gemm<false, false>(Af, Bf, d_y, (int)M, KN, OHW, KB, bias, form, alpha, st);
+}
+
+// ---- packed4: the fp4 GEMM's operands at two bits per lane (Kw a multiple of 4, as everywhere) ----
+int64_t mfma_packed4_bytes(int64_t rows, int Kw) { return ((rows + 31) / 32) * (int64_t)(Kw / 2) * 1024; }
+
+hipError_t launch_mfma_pack4(bool ternary, const int64_t* d_rows, int rows, int Kw, void* d_out, hipStream_t st) {
+    dim3 grid((rows + 31) / 32, (Kw / 4 + 3) / 4);   // 4 groups of 4 words per workgroup
+    if (grid.y > 65535) return hipErrorInvalidValue;
+    const uint32_t* R = reinterpret_cast<const uint32_t*>(d_rows);
+    if (ternary) hipLaunchKernelGGL((k_pack4<true>), grid, dim3(256), 0, st, R, rows, Kw / 4, static_cast<uint2*>(d_out));
+    else hipLaunchKernelGGL((k_pack4<false>), grid, dim3(256), 0, st, R, rows, Kw / 4, static_cast<uint2*>(d_out));
+    return hipGetLastError();
+}
+
+hipError_t launch_mfma_gemm_packed4(int type, const void* d_ac, const void* d_bc, int64_t M, int OHW, int KN, int Kw, int K_unpack,
+                                    float alpha, float* d_y, hipStream_t st) {
+    const uint4* Ac = static_cast<const uint4*>(d_ac);
+    const uint4* Bc = static_cast<const uint4*>(d_bc);
+    const int bias = type == kBNN ? 64 * Kw - K_unpack : 0;   // as launch_mfma_gemm
+    const int form = type == kTNN ? 0 : 1;
+    return OHW > 1 ? launch_gemm_p4<true>(Bc, Ac, d_y, (int)M, KN, OHW, Kw / 2, bias, form, alpha, st)
+                   : launch_gemm_p4<false>(Ac, Bc, d_y, (int)M, KN, OHW, Kw / 2, bias, form, alpha, st);
 }
 
 hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const ConvGeom& cg, int N, int KN,
@@ -916,6 +1169,15 @@ hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* 
                           int KN, int Kw, int K_unpack, float alpha, float* d_y, void* d_scratch,
                           hipStream_t st) {
     const bool a_tern = (type == kTNN || type == kTBN), b_tern = (type == kTNN || type == kBTN);
+    if (f4) {   // the fp4 GEMM takes its operands at two bits per lane
+        void* Ac = d_scratch;
+        void* Bc = static_cast<char*>(d_scratch) + mfma_packed4_bytes(M, Kw);
+        hipError_t e = launch_mfma_pack4(a_tern, d_a, (int)M, Kw, Ac, st);
+        if (e != hipSuccess) return e;
+        e = launch_mfma_pack4(b_tern, d_b, KN, Kw, Bc, st);
+        if (e != hipSuccess) return e;
+        return launch_mfma_gemm_packed4(type, Ac, Bc, M, OHW, KN, Kw, K_unpack, alpha, d_y, st);
+    }
     void* Af = d_scratch;
     void* Bf = static_cast<char*>(d_scratch) + mfma_fragment_bytes(f4, M, Kw);
     hipError_t e = launch_mfma_expand(f4, a_tern, d_a, (int)M, Kw, Af, st);

@@ -94,10 +94,11 @@ def test_engine_selection_and_scratch_sizes_need_no_device():
     # fp32 accumulation of fp4 products is exact only below 2^24 lanes: never chosen beyond
     assert lib.select_engine(0, 4096, 1, 1, 4096, 1 << 18) == lib.ENGINE_VALU
     assert lib.mm_scratch_bytes(lib.ENGINE_VALU, 0, 8192, 1, 1, 8192, 512) == 0
-    assert lib.mm_scratch_bytes(lib.ENGINE_MFMA_F4, 0, 8192, 1, 1, 8192, 512) == 2 * 256 * 512 * 1024
+    assert lib.mm_scratch_bytes(lib.ENGINE_MFMA_F4, 0, 8192, 1, 1, 8192, 512) == 2 * 256 * 256 * 1024   # two bits per lane
     assert lib.mm_scratch_bytes(lib.ENGINE_MFMA_I8, 0, 33, 1, 1, 1, 4) == (2 + 1) * 8 * 1024
-    assert lib.mm_scratch_bytes(lib.ENGINE_AUTO, 0, 8192, 1, 1, 8192, 512) == 2 * 256 * 512 * 1024
-    assert lib._L.ftnn_expand_bytes(lib.ENGINE_MFMA_F4, 100, 6) == 4 * 8 * 1024
+    assert lib.mm_scratch_bytes(lib.ENGINE_AUTO, 0, 8192, 1, 1, 8192, 512) == 2 * 256 * 256 * 1024
+    assert lib._L.ftnn_expand_bytes(lib.ENGINE_MFMA_F4, 100, 6) == 4 * 4 * 1024   # 4 row blocks x 4 pairs of K words
+    assert lib._L.ftnn_expand_bytes(lib.ENGINE_MFMA_I8, 100, 6) == 4 * 16 * 1024
     assert lib._L.ftnn_expand_bytes(lib.ENGINE_VALU, 100, 6) == 0
     # conv scratch covers either layer engine.  Vector ALU: the quantised input (16 bytes per pixel and 64
     # channels), plus dense rows and weights when C <= 32 packs several taps per word.  fp4 matrix cores: 32 bytes
