@@ -385,6 +385,15 @@ class Probe:
         return {"ms": round(r[0], 4), "lane_ops_per_s": float("%.4e" % r[1]), "frac_of_nominal": round(r[1] / (VALU_PEAK_TOPS * 1e12), 4),
                 "shader_mhz": round(r[2], 1), "lane_ops_per_lane_cycle": round(r[3], 4), "result_ok": bool(r[4])}
 
+    def mfma_rate(self, torch, trips=10000):
+        """the fp4 matrix-core chain with operands from registers (k_mfma_chain): what the chip sustains with no
+        operand traffic, and the clock it holds meanwhile"""
+        r = self._call(self.lib.probe_mfma_run, trips, torch, 4)
+        if r is None:
+            return None
+        return {"ms": round(r[0], 4), "tflops": round(r[1] / 1e12, 1), "frac_of_10100": round(r[1] / 10100e12, 4),
+                "shader_mhz": round(r[2], 1), "matrix_pipe_busy": round(r[3], 4)}
+
     def clock_after(self, torch, trips=16):
         """shader clock seen by a short, nearly idle kernel queued directly behind whatever ran last on the stream"""
         r = self._call(self.lib.probe_clock_run, trips, torch, 2)
@@ -717,7 +726,7 @@ def main():
                              "algorithmic ops = 4 per dword pair (v_or, v_bitop3, 2 x v_bcnt)"}
     mfma = {}
     for eng, key, kernel, peak in ((lib.ENGINE_MFMA_I8, "k_mfma_i8", "k_mfma<int8>", 5000.0),
-                                   (lib.ENGINE_MFMA_F4, "k_mfma_f4", "k_mfma<fp4>", 10100.0)):
+                                   (lib.ENGINE_MFMA_F4, "k_mfma_p4", "k_mfma_p4<fp4, operands at 2 bits per lane>", 10100.0)):
         ae = lib.expand_rows(eng, a, m, kw, True)
         be = lib.expand_rows(eng, b, n, kw, True)
 
@@ -736,6 +745,24 @@ def main():
         mfma[eng] = {"bound": "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "TOP/s" if eng == lib.ENGINE_MFMA_I8 else "TFLOP/s",
                      "frac": round(ach / peak, 4), "traffic": traffic, "kernel": kernel, "avg_launch_ms": round(t, 4),
                      "expand_one_operand_ms": round(te, 4)}
+        if eng == lib.ENGINE_MFMA_F4 and probe.lib is not None:
+            # registers-only chain of the same instruction, directly behind a run of the kernel
+            for _ in range(REPS):
+                gemm()
+            probe.mfma_rate(torch, 2000)
+            mfma[eng]["mfma_chain_from_registers"] = probe.mfma_rate(torch)
+        if eng == lib.ENGINE_MFMA_F4:
+            # the same launch on operands that are all zero lanes: the same instruction stream without the
+            # switching activity of real data, i.e. what the schedule alone allows when power does not bound it
+            az, bz = torch.zeros_like(ae), torch.zeros_like(be)
+
+            def gemm_zero(eng=eng, az=az, bz=bz):
+                lib.mm_expanded(eng, TNN, az, bz, m, 1, 1, n, kw, alpha, out=y)
+            gemm_zero()
+            tz = mean(event_times(torch, gemm_zero, REPS))
+            mfma[eng]["same_kernel_on_all_zero_operands"] = {"avg_launch_ms": round(tz, 4),
+                                                             "frac": round(2.0 * macs / (tz * 1e-3) / 1e12 / peak, 4)}
+            del az, bz
         if eng == auto:
             mfma[eng]["launches_timed"] = len(gemm_ms)
             mfma[eng]["timed"] = "HIP events around each GEMM launch of the timed region"

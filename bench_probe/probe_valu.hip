@@ -14,6 +14,11 @@
 //   probe_copy_run    a plain copy kernel of known size (k_probe_copy: 16 bytes per thread in, 16 bytes out): the
 //                     dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by.
 //
+//   probe_mfma_run    every wavefront of a chip-filling grid (one per SIMD, as the fp4 GEMM runs) issues nothing but
+//                     v_mfma_f32_32x32x64_f8f6f4 on E2M1 operands holding ternary codes, 16 accumulator tiles of
+//                     32 x 32 per wavefront, operands from registers: the matrix rate the chip sustains with no
+//                     operand traffic at all, and the shader clock it holds while doing so.
+//
 // All are launched on the caller's stream and timed with HIP events recorded on that stream.
 #include <hip/hip_runtime.h>
 
@@ -52,6 +57,48 @@ __global__ __launch_bounds__(256) void k_bcnt(const uint32_t* __restrict__ in, u
     if (threadIdx.x == 0) stamps[blockIdx.x] = Stamp{c0, c1, r0, r1};
 }
 
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) void k_mfma_chain(const uint4* __restrict__ in, float* __restrict__ out, int trips,
+                                                    Stamp* __restrict__ stamps) {
+    const int lane = threadIdx.x & 63;
+    v8i a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint4 u = in[(i * 64 + lane) & 511], w = in[((i + 4) * 64 + lane) & 511];
+        a[i] = v8i{(int)u.x, (int)u.y, (int)u.z, (int)u.w, 0, 0, 0, 0};
+        b[i] = v8i{(int)w.x, (int)w.y, (int)w.z, (int)w.w, 0, 0, 0, 0};
+    }
+    v16f acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+    const unsigned long long c0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+    for (int t = 0; t < trips; t++) {
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[i], b[j], acc[i][j], 4, 4, 0, 0, 0, 0);
+    }
+    const unsigned long long c1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) s += acc[i][j][e];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+    if (threadIdx.x == 0) stamps[blockIdx.x] = Stamp{c0, c1, r0, r1};
+}
+
 __global__ __launch_bounds__(256) void k_probe_copy(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n16) dst[i] = src[i];
@@ -64,6 +111,7 @@ struct State {
     int cus = 0, blocks = 0;
     double realtime_hz = 1e8;
     uint32_t host_in[1024];
+    uint4* codes = nullptr;    // 512 x 16 bytes of E2M1 ternary codes (0x2 / 0x0 / 0xA per nibble)
 } g;
 
 bool ok(hipError_t e, const char* what) {
@@ -105,6 +153,22 @@ __attribute__((visibility("default"))) int probe_valu_init(void) {
         return 1;
     for (int i = 0; i < 1024; i++) g.host_in[i] = 0x9E3779B9u * (uint32_t)(i + 1);
     if (!ok(hipMemcpy(g.in, g.host_in, sizeof g.host_in, hipMemcpyHostToDevice), "hipMemcpy")) return 1;
+    {
+        static uint32_t codes[512 * 4];
+        uint64_t x = 0x243F6A8885A308D3ull;
+        for (int i = 0; i < 512 * 4; i++) {
+            uint32_t w = 0;
+            for (int n = 0; n < 8; n++) {
+                x ^= x << 13, x ^= x >> 7, x ^= x << 17;
+                const uint32_t r = (uint32_t)(x >> 33) % 3;
+                w |= (r == 0 ? 0x0u : r == 1 ? 0x2u : 0xAu) << (4 * n);
+            }
+            codes[i] = w;
+        }
+        if (!ok(hipMalloc(&g.codes, sizeof codes), "hipMalloc") ||
+            !ok(hipMemcpy(g.codes, codes, sizeof codes, hipMemcpyHostToDevice), "hipMemcpy"))
+            return 1;
+    }
     if (!ok(hipEventCreate(&g.e0), "hipEventCreate") || !ok(hipEventCreate(&g.e1), "hipEventCreate")) return 1;
     return 0;
 }
@@ -133,6 +197,30 @@ __attribute__((visibility("default"))) int probe_valu_run(int trips, void* strea
     out[2] = mean_mhz(g.blocks);
     out[3] = out[2] > 0 ? out[1] / ((double)g.cus * 4 * 16 * out[2] * 1e6) : 0.0;
     out[4] = got == want ? 1.0 : 0.0;
+    return 0;
+}
+
+// The matrix-core chain: one workgroup of four wavefronts per compute unit, 32 fp4 MFMAs of 32 x 32 x 64 per trip
+// and wavefront.  out[0] = kernel ms, out[1] = FLOP per second (2 x 32 x 32 x 64 per MFMA), out[2] = mean shader
+// clock in MHz during the kernel, out[3] = fraction of the cycles of a SIMD at that clock in which its matrix pipe
+// was busy (32 cycles per MFMA).
+__attribute__((visibility("default"))) int probe_mfma_run(int trips, void* stream, double* out) {
+    if (probe_valu_init() != 0) return 1;
+    hipStream_t st = (hipStream_t)stream;
+    const int blocks = g.cus;
+    if (!ok(hipEventRecord(g.e0, st), "hipEventRecord")) return 1;
+    hipLaunchKernelGGL(k_mfma_chain, dim3(blocks), dim3(256), 0, st, g.codes, reinterpret_cast<float*>(g.out), trips, g.stamps);
+    if (!ok(hipGetLastError(), "launch") || !ok(hipEventRecord(g.e1, st), "hipEventRecord")) return 1;
+    if (!ok(hipMemcpyAsync(g.stamps_host, g.stamps, (size_t)blocks * sizeof(Stamp), hipMemcpyDeviceToHost, st), "copy") ||
+        !ok(hipStreamSynchronize(st), "sync"))
+        return 1;
+    float ms = 0.0f;
+    if (!ok(hipEventElapsedTime(&ms, g.e0, g.e1), "hipEventElapsedTime")) return 1;
+    const double mfmas_per_simd = 32.0 * trips;
+    out[0] = ms;
+    out[1] = mfmas_per_simd * blocks * 4 * (2.0 * 32 * 32 * 64) / (ms * 1e-3);
+    out[2] = mean_mhz(blocks);
+    out[3] = out[2] > 0 ? mfmas_per_simd * 32.0 / (ms * 1e-3 * out[2] * 1e6) : 0.0;
     return 0;
 }
 

@@ -23,7 +23,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 COPY_BYTES = 256 << 20
 
 # kernel-name fragment and grid (workgroups) -> key in the JSON; grids are those of the 8192 x 8192 x 32768 launch
-KERNELS = {"k_mfma_f4": "k_mfma<true", "k_mfma_i8": "k_mfma<false", "k_mm": "k_mm<0"}
+KERNELS = {"k_mfma_p4": "k_mfma_p4<", "k_mfma_i8": "k_mfma<false", "k_mm": "k_mm<0"}
 
 
 def per_dispatch(dirname, counter):

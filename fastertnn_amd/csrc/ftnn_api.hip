@@ -40,6 +40,8 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 // words per operand row (one plane) that every engine's 32-bit sums and offsets hold
 constexpr int kMaxRowWords = (1 << 24) - 4;
+// the fp4 GEMM sums lanes of {0, 0.5, 1}: products are multiples of 1/4, exact in fp32 while 4 * 64 * Kw <= 2^24
+constexpr int kMaxF4GemmWords = 1 << 16;
 
 // whether rows of ceil(C/64) * KH * KW words are within what 32-bit sums and offsets hold; no intermediate product
 // overflows whatever the (positive) arguments are
@@ -830,7 +832,7 @@ static int select_engine(int type, int64_t M, int KN, int Kw) {
     // measured on MI355X: from about 5 GMAC the two expansions and the matrix-core kernel (128 x 128 tiles
     // while 256 x 256 ones would leave compute units idle) take less time than the vector-ALU kernel
     const double lane_macs = (double)M * KN * 64.0 * Kw;
-    if (lane_macs >= 5e9 && KN >= 128 && 64LL * Kw < (1LL << 24)) return FTNN_ENGINE_MFMA_F4;
+    if (lane_macs >= 5e9 && KN >= 128 && Kw <= kMaxF4GemmWords) return FTNN_ENGINE_MFMA_F4;
     return FTNN_ENGINE_VALU;
 }
 
@@ -852,7 +854,7 @@ int64_t ftnn_mm_scratch_bytes(int engine, int type, int N, int OH, int OW, int K
 static int check_mfma_engine(int engine, int Kw) {
     if (engine != FTNN_ENGINE_MFMA_I8 && engine != FTNN_ENGINE_MFMA_F4)
         return fail(FTNN_EINVAL, "engine %d is not a matrix-core engine", engine);
-    if (engine == FTNN_ENGINE_MFMA_F4 && 64LL * Kw >= (1LL << 24))
+    if (engine == FTNN_ENGINE_MFMA_F4 && Kw > kMaxF4GemmWords)
         return fail(FTNN_EINVAL, "K too long for exact fp32 accumulation; use the int8 engine");
     return FTNN_OK;
 }
@@ -919,7 +921,7 @@ int ftnn_mm_engine(int engine, int type, const int64_t* d_a, const int64_t* d_b,
     if (!aligned16(d_a) || !aligned16(d_b)) return fail(FTNN_EINVAL, "GEMM operands must be 16-byte aligned");
     if (M > 0x7fffffffLL) return fail(FTNN_EINVAL, "more than 2^31-1 output rows");
     const bool f4 = engine == FTNN_ENGINE_MFMA_F4;
-    if (f4 && 64LL * Kw >= (1LL << 24))
+    if (f4 && Kw > kMaxF4GemmWords)
         return fail(FTNN_EINVAL, "K too long for exact fp32 accumulation; use the int8 engine");
     const int64_t need = ftnn_mm_scratch_bytes(engine, type, N, OH, OW, KN, K);
     if (!d_scratch || !aligned16(d_scratch) || scratch_bytes < need)

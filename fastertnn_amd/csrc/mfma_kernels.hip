@@ -321,29 +321,47 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
     store_tile<F4, SWAP, WT>(acc, Y, M, KN, OHW, prb0 + wy * WT, qrb0 + wx * WT, lane, bias, form, alpha);
 }
 
-// ------------------------------------------------- fp4 operands at two bits per lane
-// The fp4 GEMM above is bound by what it moves, not by its schedule: the stream of operand fragments from L2 into LDS
-// (8 GiB per 8192 x 8192 x 32768 launch) holds the chip's clock down.  A ternary or binary lane carries two bits of
-// information, and an E2M1 nibble of -1 / 0 / +1 uses two of its four bits: 0x2 | sign << 3, i.e. bits 1 and 3 (a
-// zero lane may keep its sign bit: -0 multiplies like +0).  Two dwords of nibbles D0, D1 therefore share one dword,
-// P = D0 | D1 >> 1, and come apart again with D0 = P & 0xAAAAAAAA, D1 = (P << 1) & 0xAAAAAAAA: 1.5 vector instructions
-// per dword, which the wavefronts issue beside their MFMAs.  Operands in this form ("packed4") are half the bytes in HBM,
-// through L2 -> LDS and through the LDS reads.
+// ------------------------------------------------- fp4 operands at two bits per lane, offset codes
+// The fp4 GEMM above is bound by power, not by its schedule.  The same instruction stream runs a quarter faster on
+// operands that are all zero, and a chain of nothing but these MFMAs on registers holds 2.39 GHz on zeros, 2.25 GHz on
+// lanes of {0, 0.5, 1} and 1.97 GHz on lanes of {-1, 0, +1}: it is the mixed signs in the adder trees and the operand
+// bytes on the move (L2 -> LDS -> registers) that hold the clock down.  The GEMM's own operand form answers both:
 //
-// Layout: 1 KiB blocks [row block of 32][pair of K words][lane l = (k half l / 32, row l % 32)][16 bytes], the 16 bytes of a
-// lane being (P0, P1) of the even K word and (P0, P1) of the odd one, P0 = D0 | D1 >> 1, P1 = D2 | D3 >> 1 with D0..D3 the
-// lane's 16 bytes of the plain fragment layout above.  One LDS-direct load of 16 bytes per lane moves a row block's two
-// K words, so a step of two K words takes half the load and half the LDS-read instructions of the plain kernel as well.
+//   offset codes   a lane a in {-1, 0, +1} travels as a' = (a + 1) / 2 in {0, 0.5, 1}, E2M1 codes 0, 1, 2: no negative
+//                  product anywhere.  With S = sum a' b' over all L = 64 Kw lanes of a row pair (padding lanes are
+//                  a = b = 0 or +-1 like any other and enter the sums below the same way)
+//                      sum a b = 4 S - sum a - sum b - L,
+//                  exact in fp32 while 4 L <= 2^24 (S is a multiple of 1/4 below L).  The row sums are counted when
+//                  the operand is packed and sit behind its blocks; the epilogue undoes the offset.
+//   two bits       codes 0, 1, 2 use bits 0 and 1 of a nibble, so two dwords of nibbles D0, D1 share one dword,
+//                  P = D0 | D1 << 2, and come apart with D0 = P & 0x33333333, D1 = (P >> 2) & 0x33333333: 1.5 vector
+//                  instructions per dword, issued beside the MFMAs.  Half the bytes in HBM, through L2 -> LDS and
+//                  through the LDS reads.
+//
+// Layout ("packed4"): 1 KiB blocks [row block of 32][pair of K words][lane l = (k half l / 32, row l % 32)][16 bytes], the
+// 16 bytes of a lane being (P0, P1) of the even K word and (P0, P1) of the odd one, P0 = D0 | D1 << 2, P1 = D2 | D3 << 2
+// with D0..D3 the lane's 16 bytes of the plain fragment layout above in offset codes.  One LDS-direct load of 16 bytes
+// per lane moves a row block's two K words.  Behind the blocks: one int32 per row (rows rounded up to 32), sum of the
+// row's lanes.
 
-// grid (row blocks, groups / 4), block 256: as k_expand<true, TERN>, writing the packed4 layout (Kw words per row)
+__global__ void k_zero_i32(int* __restrict__ p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+// grid (row blocks, groups / 4), block 256: as k_expand<true, TERN>, writing the packed4 layout (Kw words per row) and
+// adding the lanes of its rows into sums (zeroed before the launch)
 template <bool TERN>
-__global__ __launch_bounds__(256) void k_pack4(const uint32_t* __restrict__ P, int rows, int G, uint2* __restrict__ out) {
+__global__ __launch_bounds__(256) void k_pack4(const uint32_t* __restrict__ P, int rows, int G, uint2* __restrict__ out,
+                                               int* __restrict__ sums) {
     constexpr int kGPB = 4;
     constexpr int DPG = TERN ? 16 : 8;        // dwords per group and row
     constexpr int RD = kGPB * DPG;            // dwords per row in the block
     constexpr int RS = RD + 1;                // LDS row stride: odd, the 32 rows of a read hit 32 banks
     __shared__ uint32_t stage[32 * RS];
+    __shared__ int rowsum[32];
     const int rb = blockIdx.x, g0 = blockIdx.y * kGPB, t = threadIdx.x;
+    if (t < 32) rowsum[t] = 0;
     {
         constexpr int PPR = RD / 4;           // 16-byte pieces per row
         const int gmax = min(kGPB, G - g0) * (DPG / 4);
@@ -362,37 +380,84 @@ __global__ __launch_bounds__(256) void k_pack4(const uint32_t* __restrict__ P, i
     }
     __syncthreads();
     const int r = t & 31, dq = t >> 5;        // dq: dword of the group = (K word dq / 2, k half dq % 2)
-    const bool live = rb * 32 + r < rows;
+    int lanesum = 0;
 #pragma unroll
     for (int i = 0; i < kGPB; i++) {
         const int g = g0 + i;
         if (g >= G) break;
         const uint32_t sv = stage[r * RS + i * DPG + dq];
-        const uint32_t zv = TERN ? stage[r * RS + i * DPG + 8 + dq] : 0u;
-        const uint32_t nz = live ? ~zv : 0u;
-        const uint32_t s = sv & nz;
+        const uint32_t zero = TERN ? stage[r * RS + i * DPG + 8 + dq] : 0u;
+        const uint32_t plus = ~(sv | zero), minus = sv & ~zero;
+        lanesum += __popc(plus) - __popc(minus);
         uint32_t o[4];
 #pragma unroll
         for (int q = 0; q < 4; q++) {   // 8 lanes -> 8 nibbles: bit i lands on bit 4 i
-            uint32_t a = (s >> (8 * q)) & 0xffu, b = (nz >> (8 * q)) & 0xffu;
+            uint32_t a = (plus >> (8 * q)) & 0xffu, b = (zero >> (8 * q)) & 0xffu;
             a = (a | (a << 12)) & 0x000F000Fu;
             a = (a | (a << 6)) & 0x03030303u;
             a = (a | (a << 3)) & 0x11111111u;
             b = (b | (b << 12)) & 0x000F000Fu;
             b = (b | (b << 6)) & 0x03030303u;
             b = (b | (b << 3)) & 0x11111111u;
-            o[q] = (a << 3) | (b << 1);
+            o[q] = (a << 1) | b;        // +1 -> 2 (1.0), 0 -> 1 (0.5), -1 -> 0
         }
         const int w = g * 4 + (dq >> 1), h = dq & 1;   // K word and k half of this thread's 32 lanes
         const size_t block = (size_t)rb * (G * 2) + (w >> 1);
-        out[(block * 64 + h * 32 + r) * 2 + (w & 1)] = make_uint2(o[0] | (o[1] >> 1), o[2] | (o[3] >> 1));
+        out[(block * 64 + h * 32 + r) * 2 + (w & 1)] = make_uint2(o[0] | (o[1] << 2), o[2] | (o[3] << 2));
     }
+    atomicAdd(&rowsum[r], lanesum);
+    __syncthreads();
+    if (t < 32 && rb * 32 + t < rows) atomicAdd(&sums[rb * 32 + t], rowsum[t]);
 }
 
 // (P0, P1) of one K word -> the lane's 16 bytes of nibbles
 __device__ __forceinline__ uint4 unpack4(uint32_t p0, uint32_t p1) {
-    constexpr uint32_t m = 0xAAAAAAAAu;
-    return make_uint4(p0 & m, (p0 << 1) & m, p1 & m, (p1 << 1) & m);
+    constexpr uint32_t m = 0x33333333u;
+    return make_uint4(p0 & m, (p0 >> 2) & m, p1 & m, (p1 >> 2) & m);
+}
+
+// The epilogue of the offset form: dot = 4 acc - sum of the P row - sum of the Q row - lanes, then as store_tile
+// (off = lanes + the BNN bias).  sums: the tile's row sums in LDS, RB * 32 of the P side, then RB * 32 of the Q side
+// (zero for rows past the operand, which store nothing).
+template <bool SWAP, int WT>
+__device__ __forceinline__ void store_tile_offset(const Acc<true>::type (&acc)[WT][WT], float* __restrict__ Y, int M, int KN, int OHW,
+                                                  int prb, int qrb, int lane, const int* sums, int wy, int wx, int off, int form,
+                                                  float alpha) {
+    constexpr int RB = 2 * WT;
+    const bool le_form = form == 0;
+    const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN;
+#pragma unroll
+    for (int a = 0; a < WT; a++) {
+        int4 sp[4];   // the lane's 16 P rows of this block: rows 4 * (lane / 32) + 8 * j + (0..3)
+#pragma unroll
+        for (int j = 0; j < 4; j++) sp[j] = *reinterpret_cast<const int4*>(sums + (wy * WT + a) * 32 + 4 * (lane >> 5) + 8 * j);
+        const int pbase = (prb + a) * 32 + 4 * (lane >> 5);
+#pragma unroll
+        for (int b = 0; b < WT; b++) {
+            const int q = (qrb + b) * 32 + (lane & 31);
+            const bool qok = q < qrow;
+            const int sq = sums[RB * 32 + (wx * WT + b) * 32 + (lane & 31)] + off;
+            size_t qoff;
+            if (SWAP) {   // q = i is fixed per block: split it into (image, pixel) once
+                const int img = q / OHW;
+                qoff = (size_t)img * KN * OHW + (q - img * OHW);
+            } else {
+                qoff = (size_t)q;
+            }
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int p = pbase + 8 * (e >> 2) + (e & 3);
+                const int4& s4 = sp[e >> 2];
+                const int spv = (e & 3) == 0 ? s4.x : (e & 3) == 1 ? s4.y : (e & 3) == 2 ? s4.z : s4.w;
+                const int r = (int)(acc[a][b][e] * 4.0f) - spv - sq;
+                const float fr = (float)r;
+                const bool scale = le_form ? (fr <= 0.0f) : (r < 0);
+                const float f = scale ? fr * alpha : fr;
+                const size_t o = SWAP ? qoff + (size_t)p * OHW : (size_t)p * KN + qoff;
+                if (qok && p < prow) Y[o] = f;
+            }
+        }
+    }
 }
 
 // The fp4 GEMM on packed4 operands.  Same tiling as k_mfma<true, ...> (2 x 2 wavefronts, WT x WT blocks of 32 x 32 each,
@@ -402,7 +467,8 @@ __device__ __forceinline__ uint4 unpack4(uint32_t p0, uint32_t p1) {
 // and the unpacking of its first K word.
 template <bool SWAP, int WT, int kNS>
 __global__ __launch_bounds__(256) void k_mfma_p4(const uint4* __restrict__ Pc, const uint4* __restrict__ Qc, float* __restrict__ Y,
-                                                 int M, int KN, int OHW, int KP, int bias, int form, float alpha) {
+                                                 int M, int KN, int OHW, int KP, const int* __restrict__ sP,
+                                                 const int* __restrict__ sQ, int off, int form, float alpha) {
     extern __shared__ uint4 lds[];   // kNS stages of kFR KiB
     typedef typename Acc<true>::type acc_t;
     constexpr int RB = 2 * WT, kFR = 2 * RB, kFW = kFR / 4, NL = 2 * WT;   // kFW = WT blocks staged per wavefront and step
@@ -511,7 +577,16 @@ __global__ __launch_bounds__(256) void k_mfma_p4(const uint4* __restrict__ Pc, c
     for (; s + kNS < nstep; s++) step_body(s, std::true_type{});
     for (; s < nstep; s++) step_body(s, std::false_type{});
 
-    store_tile<true, SWAP, WT>(acc, Y, M, KN, OHW, prb0 + wy * WT, qrb0 + wx * WT, lane, bias, form, alpha);
+    // the tile's row sums through LDS (every load of the ring has landed and been read: the last steps wait for all)
+    __syncthreads();
+    int* sums = reinterpret_cast<int*>(lds);
+    if (tid < RB * 32) {
+        const int pr = prb0 * 32 + tid, qr = qrb0 * 32 + tid;
+        sums[tid] = pr < prow ? sP[pr] : 0;
+        sums[RB * 32 + tid] = qr < qrow ? sQ[qr] : 0;
+    }
+    __syncthreads();
+    store_tile_offset<SWAP, WT>(acc, Y, M, KN, OHW, prb0 + wy * WT, qrb0 + wx * WT, lane, sums, wy, wx, off, form, alpha);
 }
 
 // ------------------------------------------------------------ conv layer (fp4)
@@ -1003,8 +1078,8 @@ hipError_t launch_expand(bool tern, const uint32_t* rows_ptr, int rows, int G, u
 }
 
 template <bool SWAP, int WT, int NS>
-hipError_t launch_gemm_p4_tile(const uint4* Pc, const uint4* Qc, float* Y, int M, int KN, int OHW, int KP, int bias, int form,
-                               float alpha, hipStream_t st) {
+hipError_t launch_gemm_p4_tile(const uint4* Pc, const uint4* Qc, float* Y, int M, int KN, int OHW, int KP, const int* sP,
+                               const int* sQ, int off, int form, float alpha, hipStream_t st) {
     auto kern = k_mfma_p4<SWAP, WT, NS>;
     constexpr size_t lds_bytes = (size_t)NS * 4 * WT * 1024;
     // hand-counted LDS-direct loads: no scratch (see launch_gemm_tile); the opt-in to more than 64 KiB of LDS is per kernel
@@ -1020,16 +1095,16 @@ hipError_t launch_gemm_p4_tile(const uint4* Pc, const uint4* Qc, float* Y, int M
     const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN, edge = 64 * WT;
     dim3 grid((prow + edge - 1) / edge, (qrow + edge - 1) / edge);
     if (grid.y > 65535) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, st, Pc, Qc, Y, M, KN, OHW, KP, bias, form, alpha);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, st, Pc, Qc, Y, M, KN, OHW, KP, sP, sQ, off, form, alpha);
     return hipGetLastError();
 }
 
 template <bool SWAP>
-hipError_t launch_gemm_p4(const uint4* Pc, const uint4* Qc, float* Y, int M, int KN, int OHW, int KP, int bias, int form,
-                          float alpha, hipStream_t st) {
+hipError_t launch_gemm_p4(const uint4* Pc, const uint4* Qc, float* Y, int M, int KN, int OHW, int KP, const int* sP, const int* sQ,
+                          int off, int form, float alpha, hipStream_t st) {
     const int64_t big = (((int64_t)M + 255) / 256) * ((KN + 255) / 256);
-    return big < mfma_small_tile_below() ? launch_gemm_p4_tile<SWAP, 2, 4>(Pc, Qc, Y, M, KN, OHW, KP, bias, form, alpha, st)
-                                         : launch_gemm_p4_tile<SWAP, 4, 4>(Pc, Qc, Y, M, KN, OHW, KP, bias, form, alpha, st);
+    return big < mfma_small_tile_below() ? launch_gemm_p4_tile<SWAP, 2, 4>(Pc, Qc, Y, M, KN, OHW, KP, sP, sQ, off, form, alpha, st)
+                                         : launch_gemm_p4_tile<SWAP, 4, 4>(Pc, Qc, Y, M, KN, OHW, KP, sP, sQ, off, form, alpha, st);
 }
 
 }  // namespace
@@ -1065,15 +1140,23 @@ hipError_t launch_mfma_gemm(bool f4, int type, const void* d_af, const void* d_b
                 : launch_gemm<false, false>(Af, Bf, d_y, (int)M, KN, OHW, KB, bias, form, alpha, st);
 }
 
-// ---- packed4: the fp4 GEMM's operands at two bits per lane (Kw a multiple of 4, as everywhere) ----
-int64_t mfma_packed4_bytes(int64_t rows, int Kw) { return ((rows + 31) / 32) * (int64_t)(Kw / 2) * 1024; }
+// ---- packed4: the fp4 GEMM's operands at two bits per lane in offset codes (Kw a multiple of 4, as everywhere) ----
+namespace {
+inline int64_t packed4_block_bytes(int64_t rows, int Kw) { return ((rows + 31) / 32) * (int64_t)(Kw / 2) * 1024; }
+}  // namespace
+
+// the blocks, then one int32 per row of the row blocks (a multiple of 128 bytes)
+int64_t mfma_packed4_bytes(int64_t rows, int Kw) { return packed4_block_bytes(rows, Kw) + ((rows + 31) / 32) * 128; }
 
 hipError_t launch_mfma_pack4(bool ternary, const int64_t* d_rows, int rows, int Kw, void* d_out, hipStream_t st) {
     dim3 grid((rows + 31) / 32, (Kw / 4 + 3) / 4);   // 4 groups of 4 words per workgroup
     if (grid.y > 65535) return hipErrorInvalidValue;
     const uint32_t* R = reinterpret_cast<const uint32_t*>(d_rows);
-    if (ternary) hipLaunchKernelGGL((k_pack4<true>), grid, dim3(256), 0, st, R, rows, Kw / 4, static_cast<uint2*>(d_out));
-    else hipLaunchKernelGGL((k_pack4<false>), grid, dim3(256), 0, st, R, rows, Kw / 4, static_cast<uint2*>(d_out));
+    int* sums = reinterpret_cast<int*>(static_cast<char*>(d_out) + packed4_block_bytes(rows, Kw));
+    const int nsum = (int)grid.x * 32;
+    hipLaunchKernelGGL(k_zero_i32, dim3((nsum + 255) / 256), dim3(256), 0, st, sums, nsum);
+    if (ternary) hipLaunchKernelGGL((k_pack4<true>), grid, dim3(256), 0, st, R, rows, Kw / 4, static_cast<uint2*>(d_out), sums);
+    else hipLaunchKernelGGL((k_pack4<false>), grid, dim3(256), 0, st, R, rows, Kw / 4, static_cast<uint2*>(d_out), sums);
     return hipGetLastError();
 }
 
@@ -1081,10 +1164,13 @@ hipError_t launch_mfma_gemm_packed4(int type, const void* d_ac, const void* d_bc
                                     float alpha, float* d_y, hipStream_t st) {
     const uint4* Ac = static_cast<const uint4*>(d_ac);
     const uint4* Bc = static_cast<const uint4*>(d_bc);
+    const int* sA = reinterpret_cast<const int*>(static_cast<const char*>(d_ac) + packed4_block_bytes(M, Kw));
+    const int* sB = reinterpret_cast<const int*>(static_cast<const char*>(d_bc) + packed4_block_bytes(KN, Kw));
     const int bias = type == kBNN ? 64 * Kw - K_unpack : 0;   // as launch_mfma_gemm
+    const int off = 64 * Kw + bias;                           // the lanes of a row pair, padding included
     const int form = type == kTNN ? 0 : 1;
-    return OHW > 1 ? launch_gemm_p4<true>(Bc, Ac, d_y, (int)M, KN, OHW, Kw / 2, bias, form, alpha, st)
-                   : launch_gemm_p4<false>(Ac, Bc, d_y, (int)M, KN, OHW, Kw / 2, bias, form, alpha, st);
+    return OHW > 1 ? launch_gemm_p4<true>(Bc, Ac, d_y, (int)M, KN, OHW, Kw / 2, sB, sA, off, form, alpha, st)
+                   : launch_gemm_p4<false>(Ac, Bc, d_y, (int)M, KN, OHW, Kw / 2, sA, sB, off, form, alpha, st);
 }
 
 hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const ConvGeom& cg, int N, int KN,

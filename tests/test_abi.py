@@ -91,13 +91,15 @@ def test_engine_selection_and_scratch_sizes_need_no_device():
     assert lib.select_engine(0, 32, 56, 56, 64, 9) == lib.ENGINE_VALU
     assert lib.select_engine(0, 1024, 1, 1, 1024, 128) == lib.ENGINE_MFMA_F4      # the mid sizes of the reference's sweep too
     assert lib.select_engine(0, 512, 1, 1, 512, 64) == lib.ENGINE_VALU            # too little work for three launches
-    # fp32 accumulation of fp4 products is exact only below 2^24 lanes: never chosen beyond
+    # fp32 accumulation of the fp4 GEMM's products (multiples of 1/4) is exact up to 2^22 lanes: never chosen beyond
+    assert lib.select_engine(0, 4096, 1, 1, 4096, 1 << 16) == lib.ENGINE_MFMA_F4
+    assert lib.select_engine(0, 4096, 1, 1, 4096, (1 << 16) + 4) == lib.ENGINE_VALU
     assert lib.select_engine(0, 4096, 1, 1, 4096, 1 << 18) == lib.ENGINE_VALU
     assert lib.mm_scratch_bytes(lib.ENGINE_VALU, 0, 8192, 1, 1, 8192, 512) == 0
-    assert lib.mm_scratch_bytes(lib.ENGINE_MFMA_F4, 0, 8192, 1, 1, 8192, 512) == 2 * 256 * 256 * 1024   # two bits per lane
+    assert lib.mm_scratch_bytes(lib.ENGINE_MFMA_F4, 0, 8192, 1, 1, 8192, 512) == 2 * (256 * 256 * 1024 + 8192 * 4)   # two bits per lane + a sum per row
     assert lib.mm_scratch_bytes(lib.ENGINE_MFMA_I8, 0, 33, 1, 1, 1, 4) == (2 + 1) * 8 * 1024
-    assert lib.mm_scratch_bytes(lib.ENGINE_AUTO, 0, 8192, 1, 1, 8192, 512) == 2 * 256 * 256 * 1024
-    assert lib._L.ftnn_expand_bytes(lib.ENGINE_MFMA_F4, 100, 6) == 4 * 4 * 1024   # 4 row blocks x 4 pairs of K words
+    assert lib.mm_scratch_bytes(lib.ENGINE_AUTO, 0, 8192, 1, 1, 8192, 512) == 2 * (256 * 256 * 1024 + 8192 * 4)
+    assert lib._L.ftnn_expand_bytes(lib.ENGINE_MFMA_F4, 100, 6) == 4 * 4 * 1024 + 128 * 4   # 4 row blocks x 4 pairs of K words, 128 row sums
     assert lib._L.ftnn_expand_bytes(lib.ENGINE_MFMA_I8, 100, 6) == 4 * 16 * 1024
     assert lib._L.ftnn_expand_bytes(lib.ENGINE_VALU, 100, 6) == 0
     # conv scratch covers either layer engine.  Vector ALU: the quantised input (16 bytes per pixel and 64

@@ -172,7 +172,7 @@ def test_engine_argument_checks(hip):
                             None, 0, s) == 0
     torch.cuda.synchronize()
     assert hip.mm_scratch_bytes(hip.ENGINE_VALU, 0, 8192, 1, 1, 8192, 512) == 0
-    assert hip.mm_scratch_bytes(hip.ENGINE_MFMA_F4, 0, 8192, 1, 1, 8192, 512) == 2 * 256 * 256 * 1024   # two bits per lane
+    assert hip.mm_scratch_bytes(hip.ENGINE_MFMA_F4, 0, 8192, 1, 1, 8192, 512) == 2 * (256 * 256 * 1024 + 8192 * 4)   # two bits per lane + a sum per row
     assert hip.mm_scratch_bytes(hip.ENGINE_MFMA_I8, 0, 33, 1, 1, 1, 4) == (2 + 1) * 8 * 1024
     assert hip.select_engine(0, 8192, 1, 1, 8192, 512) == hip.ENGINE_MFMA_F4
     assert hip.select_engine(0, 1, 56, 56, 256, 36) == hip.ENGINE_VALU
