@@ -58,6 +58,9 @@ def parse():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 256 MiB device copy, the known-size dispatch that "
                          "FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
+    ap.add_argument("--chain-codes", action="store_true",
+                    help="run the registers-only MFMA chain on every code table of the probe (lane content against "
+                         "clock), not only the two the GEMM's history needs")
     return ap.parse_args()
 
 
@@ -385,12 +388,17 @@ class Probe:
         return {"ms": round(r[0], 4), "lane_ops_per_s": float("%.4e" % r[1]), "frac_of_nominal": round(r[1] / (VALU_PEAK_TOPS * 1e12), 4),
                 "shader_mhz": round(r[2], 1), "lane_ops_per_lane_cycle": round(r[3], 4), "result_ok": bool(r[4])}
 
-    def mfma_rate(self, torch, trips=10000):
-        """the fp4 matrix-core chain with operands from registers (k_mfma_chain): what the chip sustains with no
-        operand traffic, and the clock it holds meanwhile"""
-        r = self._call(self.lib.probe_mfma_run, trips, torch, 4)
-        if r is None:
+    MFMA_CHAIN_FORMS = ("lanes_as_minus1_0_plus1", "lanes_as_0_half_1", "all_zero", "lanes_as_0_0_1", "lanes_as_0_1_2",
+                        "lanes_as_minus1.5_0_plus1.5", "lanes_as_minus6_0_plus6")
+
+    def mfma_rate(self, torch, form, trips=10000):
+        """the fp4 matrix-core chain with operands from registers (k_mfma_chain) on uniformly random ternary lanes
+        coded by table `form` (index into MFMA_CHAIN_FORMS; 0 = -1 / 0 / +1, 1 = the GEMM's offset codes 0 / 0.5 / 1):
+        what the chip sustains with no operand traffic, and the clock it holds meanwhile"""
+        out = (self.C.c_double * 4)()
+        if self.lib.probe_mfma_run(int(trips), int(form), self.C.c_void_p(torch.cuda.current_stream().cuda_stream), out) != 0:
             return None
+        r = list(out)
         return {"ms": round(r[0], 4), "tflops": round(r[1] / 1e12, 1), "frac_of_10100": round(r[1] / 10100e12, 4),
                 "shader_mhz": round(r[2], 1), "matrix_pipe_busy": round(r[3], 4)}
 
@@ -745,15 +753,9 @@ def main():
         mfma[eng] = {"bound": "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "TOP/s" if eng == lib.ENGINE_MFMA_I8 else "TFLOP/s",
                      "frac": round(ach / peak, 4), "traffic": traffic, "kernel": kernel, "avg_launch_ms": round(t, 4),
                      "expand_one_operand_ms": round(te, 4)}
-        if eng == lib.ENGINE_MFMA_F4 and probe.lib is not None:
-            # registers-only chain of the same instruction, directly behind a run of the kernel
-            for _ in range(REPS):
-                gemm()
-            probe.mfma_rate(torch, 2000)
-            mfma[eng]["mfma_chain_from_registers"] = probe.mfma_rate(torch)
         if eng == lib.ENGINE_MFMA_F4:
-            # the same launch on operands that are all zero lanes: the same instruction stream without the
-            # switching activity of real data, i.e. what the schedule alone allows when power does not bound it
+            # the same launch on operand buffers of all-zero codes: the same instruction stream without the switching
+            # activity of real data, i.e. what the schedule alone allows when power does not bound it
             az, bz = torch.zeros_like(ae), torch.zeros_like(be)
 
             def gemm_zero(eng=eng, az=az, bz=bz):
@@ -763,6 +765,14 @@ def main():
             mfma[eng]["same_kernel_on_all_zero_operands"] = {"avg_launch_ms": round(tz, 4),
                                                              "frac": round(2.0 * macs / (tz * 1e-3) / 1e12 / peak, 4)}
             del az, bz
+        if eng == lib.ENGINE_MFMA_F4 and probe.lib is not None:
+            # registers-only chain of the same instruction, directly behind a run of the kernel
+            for _ in range(REPS):
+                gemm()
+            mfma[eng]["mfma_chain_from_registers"] = {}
+            for form in ((1, 0) if not args.chain_codes else range(len(Probe.MFMA_CHAIN_FORMS))):
+                probe.mfma_rate(torch, form, 2000)
+                mfma[eng]["mfma_chain_from_registers"][Probe.MFMA_CHAIN_FORMS[form]] = probe.mfma_rate(torch, form)
         if eng == auto:
             mfma[eng]["launches_timed"] = len(gemm_ms)
             mfma[eng]["timed"] = "HIP events around each GEMM launch of the timed region"

@@ -15,9 +15,11 @@
 //                     dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by.
 //
 //   probe_mfma_run    every wavefront of a chip-filling grid (one per SIMD, as the fp4 GEMM runs) issues nothing but
-//                     v_mfma_f32_32x32x64_f8f6f4 on E2M1 operands holding ternary codes, 16 accumulator tiles of
-//                     32 x 32 per wavefront, operands from registers: the matrix rate the chip sustains with no
-//                     operand traffic at all, and the shader clock it holds while doing so.
+//                     v_mfma_f32_32x32x64_f8f6f4 on E2M1 operands holding uniformly random ternary lanes, 16
+//                     accumulator tiles of 32 x 32 per wavefront, operands from registers: the matrix rate the chip
+//                     sustains with no operand traffic at all, and the shader clock it holds while doing so.  The
+//                     lanes are coded either as -1 / 0 / +1 (codes 0xA, 0x0, 0x2) or offset as 0 / 0.5 / 1 (codes
+//                     0, 1, 2, the form the GEMM's operands travel in): the clock differs between the two.
 //
 // All are launched on the caller's stream and timed with HIP events recorded on that stream.
 #include <hip/hip_runtime.h>
@@ -29,6 +31,13 @@ namespace {
 
 constexpr int kAcc = 8;      // independent accumulators per lane
 constexpr int kUnroll = 64;  // popcounts per accumulator and loop trip: 512 vector instructions per 3 scalar ones of loop control
+
+// E2M1 codes of a lane that is -1, 0, +1, by table: 0 the plain codes, 1 the offset codes (a + 1) / 2 the GEMM's operands
+// travel in; the others only show how the clock depends on the lanes' content: 2 all zero, 3 {0, +1}, 4 {0, 1, 2},
+// 5 {-1.5, 0, +1.5}, 6 {-6, 0, +6}
+constexpr int kForms = 7;
+constexpr uint32_t kCode[kForms][3] = {{0xA, 0x0, 0x2}, {0x0, 0x1, 0x2}, {0x0, 0x0, 0x0}, {0x0, 0x0, 0x2},
+                                       {0x0, 0x2, 0x4}, {0xB, 0x0, 0x3}, {0xF, 0x0, 0x7}};
 
 struct Stamp {
     unsigned long long clk0, clk1, rt0, rt1;
@@ -111,7 +120,7 @@ struct State {
     int cus = 0, blocks = 0;
     double realtime_hz = 1e8;
     uint32_t host_in[1024];
-    uint4* codes = nullptr;    // 512 x 16 bytes of E2M1 ternary codes (0x2 / 0x0 / 0xA per nibble)
+    uint4* codes[kForms] = {};    // 512 x 16 bytes of E2M1 nibbles per code table (kCode)
 } g;
 
 bool ok(hipError_t e, const char* what) {
@@ -153,20 +162,19 @@ __attribute__((visibility("default"))) int probe_valu_init(void) {
         return 1;
     for (int i = 0; i < 1024; i++) g.host_in[i] = 0x9E3779B9u * (uint32_t)(i + 1);
     if (!ok(hipMemcpy(g.in, g.host_in, sizeof g.host_in, hipMemcpyHostToDevice), "hipMemcpy")) return 1;
-    {
+    for (int form = 0; form < kForms; form++) {
         static uint32_t codes[512 * 4];
         uint64_t x = 0x243F6A8885A308D3ull;
         for (int i = 0; i < 512 * 4; i++) {
             uint32_t w = 0;
             for (int n = 0; n < 8; n++) {
                 x ^= x << 13, x ^= x >> 7, x ^= x << 17;
-                const uint32_t r = (uint32_t)(x >> 33) % 3;
-                w |= (r == 0 ? 0x0u : r == 1 ? 0x2u : 0xAu) << (4 * n);
+                w |= kCode[form][(uint32_t)(x >> 33) % 3] << (4 * n);
             }
             codes[i] = w;
         }
-        if (!ok(hipMalloc(&g.codes, sizeof codes), "hipMalloc") ||
-            !ok(hipMemcpy(g.codes, codes, sizeof codes, hipMemcpyHostToDevice), "hipMemcpy"))
+        if (!ok(hipMalloc(&g.codes[form], sizeof codes), "hipMalloc") ||
+            !ok(hipMemcpy(g.codes[form], codes, sizeof codes, hipMemcpyHostToDevice), "hipMemcpy"))
             return 1;
     }
     if (!ok(hipEventCreate(&g.e0), "hipEventCreate") || !ok(hipEventCreate(&g.e1), "hipEventCreate")) return 1;
@@ -203,13 +211,13 @@ __attribute__((visibility("default"))) int probe_valu_run(int trips, void* strea
 // The matrix-core chain: one workgroup of four wavefronts per compute unit, 32 fp4 MFMAs of 32 x 32 x 64 per trip
 // and wavefront.  out[0] = kernel ms, out[1] = FLOP per second (2 x 32 x 32 x 64 per MFMA), out[2] = mean shader
 // clock in MHz during the kernel, out[3] = fraction of the cycles of a SIMD at that clock in which its matrix pipe
-// was busy (32 cycles per MFMA).
-__attribute__((visibility("default"))) int probe_mfma_run(int trips, void* stream, double* out) {
-    if (probe_valu_init() != 0) return 1;
+// was busy (32 cycles per MFMA).  form: the code table of the lanes (kCode): 0 = -1 / 0 / +1, 1 = 0 / 0.5 / 1, ...
+__attribute__((visibility("default"))) int probe_mfma_run(int trips, int form, void* stream, double* out) {
+    if (probe_valu_init() != 0 || form < 0 || form >= kForms) return 1;
     hipStream_t st = (hipStream_t)stream;
     const int blocks = g.cus;
     if (!ok(hipEventRecord(g.e0, st), "hipEventRecord")) return 1;
-    hipLaunchKernelGGL(k_mfma_chain, dim3(blocks), dim3(256), 0, st, g.codes, reinterpret_cast<float*>(g.out), trips, g.stamps);
+    hipLaunchKernelGGL(k_mfma_chain, dim3(blocks), dim3(256), 0, st, g.codes[form], reinterpret_cast<float*>(g.out), trips, g.stamps);
     if (!ok(hipGetLastError(), "launch") || !ok(hipEventRecord(g.e1, st), "hipEventRecord")) return 1;
     if (!ok(hipMemcpyAsync(g.stamps_host, g.stamps, (size_t)blocks * sizeof(Stamp), hipMemcpyDeviceToHost, st), "copy") ||
         !ok(hipStreamSynchronize(st), "sync"))

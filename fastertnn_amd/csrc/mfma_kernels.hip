@@ -344,9 +344,11 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
 // per lane moves a row block's two K words.  Behind the blocks: one int32 per row (rows rounded up to 32), sum of the
 // row's lanes.
 
-__global__ void k_zero_i32(int* __restrict__ p, int n) {
+// zeroes p[0 .. n) and q[0 .. m) (m may be 0)
+__global__ void k_zero_i32(int* __restrict__ p, int n, int* __restrict__ q, int m) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0;
+    else if (i - n < m) q[i - n] = 0;
 }
 
 // grid (row blocks, groups / 4), block 256: as k_expand<true, TERN>, writing the packed4 layout (Kw words per row) and
@@ -1148,16 +1150,27 @@ inline int64_t packed4_block_bytes(int64_t rows, int Kw) { return ((rows + 31) /
 // the blocks, then one int32 per row of the row blocks (a multiple of 128 bytes)
 int64_t mfma_packed4_bytes(int64_t rows, int Kw) { return packed4_block_bytes(rows, Kw) + ((rows + 31) / 32) * 128; }
 
-hipError_t launch_mfma_pack4(bool ternary, const int64_t* d_rows, int rows, int Kw, void* d_out, hipStream_t st) {
+namespace {
+inline int* packed4_sums(void* d_out, int64_t rows, int Kw) {
+    return reinterpret_cast<int*>(static_cast<char*>(d_out) + packed4_block_bytes(rows, Kw));
+}
+
+// zero_sums = false: the caller has zeroed the row sums on the stream already
+hipError_t launch_pack4(bool ternary, const int64_t* d_rows, int rows, int Kw, void* d_out, bool zero_sums, hipStream_t st) {
     dim3 grid((rows + 31) / 32, (Kw / 4 + 3) / 4);   // 4 groups of 4 words per workgroup
     if (grid.y > 65535) return hipErrorInvalidValue;
     const uint32_t* R = reinterpret_cast<const uint32_t*>(d_rows);
-    int* sums = reinterpret_cast<int*>(static_cast<char*>(d_out) + packed4_block_bytes(rows, Kw));
+    int* sums = packed4_sums(d_out, rows, Kw);
     const int nsum = (int)grid.x * 32;
-    hipLaunchKernelGGL(k_zero_i32, dim3((nsum + 255) / 256), dim3(256), 0, st, sums, nsum);
+    if (zero_sums) hipLaunchKernelGGL(k_zero_i32, dim3((nsum + 255) / 256), dim3(256), 0, st, sums, nsum, nullptr, 0);
     if (ternary) hipLaunchKernelGGL((k_pack4<true>), grid, dim3(256), 0, st, R, rows, Kw / 4, static_cast<uint2*>(d_out), sums);
     else hipLaunchKernelGGL((k_pack4<false>), grid, dim3(256), 0, st, R, rows, Kw / 4, static_cast<uint2*>(d_out), sums);
     return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_mfma_pack4(bool ternary, const int64_t* d_rows, int rows, int Kw, void* d_out, hipStream_t st) {
+    return launch_pack4(ternary, d_rows, rows, Kw, d_out, true, st);
 }
 
 hipError_t launch_mfma_gemm_packed4(int type, const void* d_ac, const void* d_bc, int64_t M, int OHW, int KN, int Kw, int K_unpack,
@@ -1258,9 +1271,12 @@ hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* 
     if (f4) {   // the fp4 GEMM takes its operands at two bits per lane
         void* Ac = d_scratch;
         void* Bc = static_cast<char*>(d_scratch) + mfma_packed4_bytes(M, Kw);
-        hipError_t e = launch_mfma_pack4(a_tern, d_a, (int)M, Kw, Ac, st);
+        const int na = (int)((M + 31) / 32) * 32, nb = (KN + 31) / 32 * 32;   // one launch zeroes both operands' row sums
+        hipLaunchKernelGGL(k_zero_i32, dim3((na + nb + 255) / 256), dim3(256), 0, st, packed4_sums(Ac, M, Kw), na,
+                           packed4_sums(Bc, KN, Kw), nb);
+        hipError_t e = launch_pack4(a_tern, d_a, (int)M, Kw, Ac, false, st);
         if (e != hipSuccess) return e;
-        e = launch_mfma_pack4(b_tern, d_b, KN, Kw, Bc, st);
+        e = launch_pack4(b_tern, d_b, KN, Kw, Bc, false, st);
         if (e != hipSuccess) return e;
         return launch_mfma_gemm_packed4(type, Ac, Bc, M, OHW, KN, Kw, K_unpack, alpha, d_y, st);
     }

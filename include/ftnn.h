@@ -165,7 +165,7 @@ FTNN_API int ftnn_mm(int type, const int64_t *d_a, const int64_t *d_b, int N, in
 #define FTNN_ENGINE_AUTO 0
 #define FTNN_ENGINE_VALU 1    /* bit-plane popcount on the vector ALU, no scratch   */
 #define FTNN_ENGINE_MFMA_I8 2 /* v_mfma_i32_32x32x32_i8 on expanded operands         */
-#define FTNN_ENGINE_MFMA_F4 3 /* v_mfma_f32_32x32x64_f8f6f4 (fp4) on expanded operands */
+#define FTNN_ENGINE_MFMA_F4 3 /* v_mfma_f32_32x32x64_f8f6f4 (fp4); GEMM rows of at most 65536 words */
 
 /* the engine FTNN_ENGINE_AUTO resolves to for this shape (never AUTO) */
 FTNN_API int ftnn_select_engine(int type, int N, int OH, int OW, int KN, int K);
@@ -189,6 +189,9 @@ FTNN_API int ftnn_mm_engine(int engine, int type, const int64_t *d_a, const int6
  * plane (ternary != 0: Packing-2, else single-plane binary) into the operand format of
  * `engine` (FTNN_ENGINE_MFMA_I8 or _F4), ftnn_expand_bytes() bytes at d_out;
  * ftnn_mm_expanded multiplies two expanded operands and applies PReLU like ftnn_mm.
+ * The fp4 format is opaque: two bits per lane, lane a stored as (a + 1) / 2, followed by
+ * one int32 per row with the sum of the row's lanes (the GEMM undoes the offset with it);
+ * its sums are exact in fp32 for K <= 65536 words, longer rows are refused (use int8).
  * No counterpart in the reference.
  */
 FTNN_API int64_t ftnn_expand_bytes(int engine, int rows, int K);

@@ -156,6 +156,46 @@ def test_lanes_flagged_zero_and_negative_count_as_zero(hip, oracle):
         assert got.tobytes() == want.tobytes(), "engine %d" % eng
 
 
+def test_fp4_gemm_is_exact_on_its_longest_rows(hip):
+    """The fp4 GEMM sums lanes coded (a + 1) / 2 in fp32: quarters up to the lane count, exact up to 65536 words per row.
+    Rows of that length, almost all lanes +1 on both sides (sums just below 2^22, where fp32 resolves 1/4 and no
+    less), against the vector-ALU engine and against numpy on the bit planes."""
+    import torch
+    rng = np.random.default_rng(11)
+    m, n, kw = 40, 33, 1 << 16
+
+    def sparse(shape):
+        r = rng.integers(-2 ** 63, 2 ** 63, size=(5,) + shape, dtype=np.int64)
+        return r[0] & r[1] & r[2] & r[3] & r[4]
+
+    def operand(rows):
+        v = np.empty((rows, kw // 4, 2, 4), dtype=np.int64)
+        v[:, :, 0, :] = sparse((rows, kw // 4, 4))     # sign bits: 1 lane in 32 negative
+        v[:, :, 1, :] = sparse((rows, kw // 4, 4))     # zero bits: 1 lane in 32 zero
+        return v
+    a, b = operand(m), operand(n)
+    print("case longest fp4 rows", m, n, kw, flush=True)
+    a_d, b_d = _dev(a.reshape(-1)), _dev(b.reshape(-1))
+    want = hip.mm_engine(hip.ENGINE_VALU, TNN, a_d, b_d, m, 1, 1, n, kw, 0.5).cpu().numpy()
+    got = hip.mm_engine(hip.ENGINE_MFMA_F4, TNN, a_d, b_d, m, 1, 1, n, kw, 0.5).cpu().numpy()
+    assert got.tobytes() == want.tobytes()
+    # numpy on the planes for a few (row, column) pairs: sum over lanes of a * b
+    pop = lambda x: int(np.unpackbits(x.view(np.uint8)).sum())
+    for i, j in ((0, 0), (39, 32), (17, 5)):
+        sa, za, sb, zb = a[i, :, 0, :], a[i, :, 1, :], b[j, :, 0, :], b[j, :, 1, :]
+        nz = ~(za | zb)
+        dot = pop(nz) - 2 * pop((sa ^ sb) & nz)
+        assert dot > 3_000_000                       # the case is near the top of the range
+        assert got.reshape(m, n)[i, j] == np.float32(dot)
+    # one group of words more is refused, and AUTO does not pick the engine there
+    L, s = hip._L, hip._stream()
+    y = torch.empty(16, device="cuda")
+    assert L.ftnn_mm_engine(hip.ENGINE_MFMA_F4, 0, a_d.data_ptr(), b_d.data_ptr(), 1, 1, 1, 1, kw + 4, 0, 0.5, y.data_ptr(),
+                            a_d.data_ptr(), 1 << 20, s) == -1
+    assert b"too long" in L.ftnn_last_error()
+    assert hip.select_engine(0, 4096, 1, 1, 4096, kw + 4) == hip.ENGINE_VALU
+
+
 def test_engine_argument_checks(hip):
     import torch
     a = torch.zeros(64 * 8, dtype=torch.int64, device="cuda")
