@@ -129,6 +129,26 @@ def cpu_gemm_baseline(a_host, b_host, rows, n, kw, alpha):
     return y, dt, kind
 
 
+def graph_times(torch, fn, y, reps, n_graph=10):
+    """device time of `fn` with no host in the loop: n_graph calls recorded into one graph, HIP events around its
+    replay, per call; every replay must leave in y what the eager call left there (returns ms, same_bits)"""
+    fn()
+    torch.cuda.synchronize()
+    y_eager = y.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(n_graph):
+            fn()
+    y.zero_()
+    graph.replay()
+    torch.cuda.synchronize()
+    same = bool(torch.equal(y, y_eager))
+    ms = sorted(event_times(torch, graph.replay, reps))[reps // 2] / n_graph
+    same = same and bool(torch.equal(y, y_eager))
+    del graph
+    return ms, same
+
+
 def small_gemm(torch, lib, m, n, k, reps=30):
     """the reference's own CPU-runnable GEMM case on every engine (whole call, HIP events), the
     host entry point mm_tnn (host pointers in and out) and the CPU reference on one core"""
@@ -156,8 +176,10 @@ def small_gemm(torch, lib, m, n, k, reps=30):
         run()
         t = event_times(torch, run, reps)
         t = sum(t) / len(t)
-        out[name] = {"call_ms": round(t, 4), "gmacs": round(float(m) * n * k / t / 1e6, 1),
-                     "bit_exact_vs_cpu": bool(y.cpu().numpy().tobytes() == np.ascontiguousarray(want).tobytes())}
+        exact = bool(y.cpu().numpy().tobytes() == np.ascontiguousarray(want).tobytes())
+        tg, same = graph_times(torch, run, y, reps)
+        out[name] = {"call_ms": round(t, 4), "gmacs": round(float(m) * n * k / t / 1e6, 1), "bit_exact_vs_cpu": exact,
+                     "device_ms_in_a_graph_of_10_calls": round(tg, 4), "graph_replays_same_bits_as_eager": same}
     t_abi = []
     for _ in range(10):
         t0 = time.perf_counter()
@@ -264,8 +286,12 @@ def conv_latency(torch, lib, typ, shape, batch, seed, reps=20):
     for _ in range(3):
         step()
         step_rows()
-    kernel_ms = sorted(event_times(torch, step, reps))[reps // 2]
+    call_ms = sorted(event_times(torch, step, reps))[reps // 2]
     rows_ms = sorted(event_times(torch, step_rows, reps))[reps // 2]
+    # device time of the layer with no host in the loop (a single call issued from Python leaves the device idle
+    # between its two launches)
+    n_graph = 10
+    kernel_ms, graph_same = graph_times(torch, step, y, reps, n_graph)
     xh, thrh, qwh = x.cpu().numpy(), thr.cpu().numpy(), qw.cpu().numpy()
     yh = lib.host_conv(typ, xh, thrh, qwh, kn, kh, kw, pad, stride, 0.5)
     # ABI-inclusive: the C call tnns_conv alone, host pointers in, malloc'd host pointer out (freed as a C caller would)
@@ -279,7 +305,10 @@ def conv_latency(torch, lib, typ, shape, batch, seed, reps=20):
         lib._L.tnns_conv(ctypes.byref(tc))
         t.append((time.perf_counter() - t0) * 1e3)
         lib._libc.free(tc.output)
-    out = {"kernel_ms": round(kernel_ms, 4), "kernel_ms_from_packed_rows": round(rows_ms, 4),
+    out = {"kernel_ms": round(kernel_ms, 4),
+           "kernel_ms_is": "HIP events around a graph replay of %d calls (weights prepared), per call" % n_graph,
+           "graph_replays_same_bits_as_eager": graph_same,
+           "single_call_ms_from_python": round(call_ms, 4), "single_call_ms_from_packed_rows": round(rows_ms, 4),
            "engine": lib.ENGINE_NAMES[lib.select_conv_engine(typ, batch, c, ih, iw, kn, kh, kw, pad, stride)],
            "abi_ms": round(sorted(t)[7], 3),
            "gmacs_kernel": round(batch * oh * ow * kn * c * kh * kw / kernel_ms / 1e6, 1)}
