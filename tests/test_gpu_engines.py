@@ -125,6 +125,29 @@ def test_matrix_core_engines_with_256x256_tiles(hip, oracle, typ, shape):
 
 
 @pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
+def test_weights_kept_in_engine_form_serve_every_batch(hip, oracle, typ):
+    """ftnn_expand_rows once for the weights, then ftnn_mm_expanded for activations of several sizes: few rows (128 x 128
+    tiles), many rows (256 x 256 tiles), a conv-shaped result; the engine form of an operand must not depend on the
+    other operand or on the tiling that a call picks.  Both matrix-core engines, ragged everywhere, K tail."""
+    kn, kw = 2700, 8
+    ku = 64 * kw - 5
+    rng = np.random.default_rng(300 + typ)
+    at, wt = act_is_ternary(typ), weight_is_ternary(typ)
+    b = rng.integers(-2 ** 63, 2 ** 63, size=kn * kw * (2 if wt else 1), dtype=np.int64)
+    b_d = _dev(b)
+    for eng in (hip.ENGINE_MFMA_I8, hip.ENGINE_MFMA_F4):
+        b_exp = hip.expand_rows(eng, b_d, kn, kw, wt)
+        for n, oh, ow in ((70, 1, 1), (3700, 1, 1), (3, 37, 35)):
+            m = n * oh * ow
+            print("case", TYPE_NAMES[typ], "engine", eng, "rows", m, flush=True)
+            a = rng.integers(-2 ** 63, 2 ** 63, size=m * kw * (2 if at else 1), dtype=np.int64)
+            want = oracle.mm(typ, a, b, n, oh, ow, kn, kw, -0.5, ku)
+            a_exp = hip.expand_rows(eng, _dev(a), m, kw, at)
+            got = hip.mm_expanded(eng, typ, a_exp, b_exp, n, oh, ow, kn, kw, -0.5, ku).cpu().numpy()
+            assert got.tobytes() == want.tobytes(), "engine %d rows %d" % (eng, m)
+
+
+@pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
 @pytest.mark.parametrize("shape", [(4200, 1, 1, 1100, 4), (7, 30, 29, 1070, 8)], ids=["row_major", "nchw"])
 def test_vector_alu_gemm_walks_large_grids_in_panels(hip, oracle, typ, shape):
     """grids of 32 x 32 workgroups and more are renumbered into panels of 32 row tiles (the last one narrower when the
