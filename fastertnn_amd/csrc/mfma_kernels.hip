@@ -8,9 +8,11 @@
 //     accumulate;
 //   * MFMA fp4   (v_mfma_f32_32x32x64_f8f6f4, E2M1): lanes become nibbles 0x2 / 0x0 / 0xA
 //     (+1.0 / 0 / -1.0), fp32 accumulate -- exact while 64*Kw < 2^24, which the host
-//     checks.  Twice the matrix rate of int8 and half the operand bytes.
+//     checks.  Twice the matrix rate of int8 and half the operand bytes.  This is the form
+//     of the conv layer kernels and their prepared weights; the fp4 GEMM engine itself
+//     (k_pack4, k_mfma_p4 further down) codes a lane a as (a + 1) / 2 at two bits per lane.
 //
-// Two kernels:
+// The kernels of the int8 engine and of the layers' GEMM route:
 //   k_expand  Packing-2 (or single-plane binary) rows -> "fragments": 1 KiB blocks
 //             holding 32 rows x 32 (int8) or 64 (fp4) lanes in exactly the register
 //             layout of an MFMA operand (lane l = (k half l/32, row l%32), 16 bytes).
