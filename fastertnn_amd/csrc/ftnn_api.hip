@@ -847,7 +847,7 @@ int64_t ftnn_mm_scratch_bytes(int engine, int type, int N, int OH, int OW, int K
     const int Kw = round4(K);
     if (engine == FTNN_ENGINE_AUTO) engine = select_engine(type, M, KN, Kw);
     if (engine != FTNN_ENGINE_MFMA_I8 && engine != FTNN_ENGINE_MFMA_F4) return 0;
-    if (engine == FTNN_ENGINE_MFMA_F4) return mfma_packed4_bytes(M, Kw) + mfma_packed4_bytes(KN, Kw);
+    if (engine == FTNN_ENGINE_MFMA_F4) return mfma_f4_mm_scratch_bytes(M, KN, Kw);
     return mfma_fragment_bytes(false, M, Kw) + mfma_fragment_bytes(false, KN, Kw);
 }
 

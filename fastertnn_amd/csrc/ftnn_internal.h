@@ -260,6 +260,8 @@ int64_t mfma_packed4_bytes(int64_t rows, int Kw);
 hipError_t launch_mfma_pack4(bool ternary, const int64_t* d_rows, int rows, int Kw, void* d_out, hipStream_t st);
 hipError_t launch_mfma_gemm_packed4(int type, const void* d_ac, const void* d_bc, int64_t M, int OHW, int KN, int Kw, int K_unpack,
                                     float alpha, float* d_y, hipStream_t st);
+// scratch of launch_mm_mfma on the fp4 engine (it picks the operand form by shape)
+int64_t mfma_f4_mm_scratch_bytes(int64_t M, int KN, int Kw);
 hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* d_b, int64_t M, int OHW,
                           int KN, int Kw, int K_unpack, float alpha, float* d_y, void* d_scratch,
                           hipStream_t st);

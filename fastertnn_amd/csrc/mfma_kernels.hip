@@ -1266,11 +1266,24 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
     return by_mode(std::true_type{}, std::false_type{});   // BTN, BNN
 }
 
+// A whole call from packed rows expands both operands itself, so it may pick the operand form by shape: problems on
+// 128 x 128 tiles (few tiles; one workgroup per compute unit, nothing to hide the read -> unpack -> multiply chain of the
+// packed4 kernel's short steps) run faster on plain fp4 fragments (2048 x 2048 x 16384: 54 against 62 us, 1024 x 1024 x
+// 8192: 30 against 36), the large ones on packed4 in offset codes.
+static bool f4_whole_call_plain(int64_t M, int KN) {
+    return ((M + 255) / 256) * ((KN + 255) / 256) < mfma_small_tile_below();
+}
+
+int64_t mfma_f4_mm_scratch_bytes(int64_t M, int KN, int Kw) {
+    return f4_whole_call_plain(M, KN) ? mfma_fragment_bytes(true, M, Kw) + mfma_fragment_bytes(true, KN, Kw)
+                                      : mfma_packed4_bytes(M, Kw) + mfma_packed4_bytes(KN, Kw);
+}
+
 hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* d_b, int64_t M, int OHW,
                           int KN, int Kw, int K_unpack, float alpha, float* d_y, void* d_scratch,
                           hipStream_t st) {
     const bool a_tern = (type == kTNN || type == kTBN), b_tern = (type == kTNN || type == kBTN);
-    if (f4) {   // the fp4 GEMM takes its operands at two bits per lane
+    if (f4 && !f4_whole_call_plain(M, KN)) {   // the fp4 GEMM takes its operands at two bits per lane
         void* Ac = d_scratch;
         void* Bc = static_cast<char*>(d_scratch) + mfma_packed4_bytes(M, Kw);
         const int na = (int)((M + 31) / 32) * 32, nb = (KN + 31) / 32 * 32;   // one launch zeroes both operands' row sums
