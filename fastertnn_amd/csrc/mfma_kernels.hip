@@ -467,8 +467,9 @@ __device__ __forceinline__ void store_tile_offset(const Acc<true>::type (&acc)[W
 // The fp4 GEMM on packed4 operands.  Same tiling as k_mfma<true, ...> (2 x 2 wavefronts, WT x WT blocks of 32 x 32 each,
 // steps of two K words, ring of kNS stages filled by LDS-direct loads that the kernel counts by hand), with one 1 KiB block
 // per row block and step.  A step: the first K word's 16 multiplies run while the second one's operands are unpacked;
-// then the barrier; the second K word's multiplies run beside the loads of stage s + kNS, the LDS reads of stage s + 1
-// and the unpacking of its first K word.
+// then the barrier; the second K word's multiplies run beside the loads of stage s + kNS and the LDS reads of stage
+// s + 1, one read per slot of two multiplies (a 16-byte LDS read holds the wavefront's issue for 16 cycles), each block
+// unpacked LAG slots after its read -- the last LAG blocks in the first slots of the next step.
 template <bool SWAP, int WT, int kNS>
 __global__ __launch_bounds__(256) void k_mfma_p4(const uint4* __restrict__ Pc, const uint4* __restrict__ Qc, float* __restrict__ Y,
                                                  int M, int KN, int OHW, int KP, const int* __restrict__ sP,
@@ -543,11 +544,18 @@ __global__ __launch_bounds__(256) void k_mfma_p4(const uint4* __restrict__ Pc, c
 #pragma unroll
     for (int i = 0; i < NL; i++) unpack(0, i);
 
+    // slots between the LDS read of a block and its unpacking: far enough for the read to have landed, near enough for
+    // every block to be unpacked by the slot that multiplies it first (block b: slot 0 for P block 0, (b - 1) / (WT / 2)
+    // for Q block b - 1, 2 (b - WT) for P block b - WT)
+    constexpr int LAG = WT >= 4 ? 4 : 3;
+    static_assert(LAG <= NL - 1 && LAG <= NL - WT + (WT - 1) / (WT / 2) && LAG <= WT + 1, "a block is unpacked before its first multiply");
     auto step_body = [&](int s, auto full_tag) {
         constexpr bool FULL = decltype(full_tag)::value;   // FULL: s + kNS < nstep
-        // first K word: multiply, and unpack the second one's operands (their packed blocks arrived a phase ago)
+        // first K word: multiply, and unpack the second one's operands (their packed blocks arrived a phase ago); the
+        // first LAG slots also unpack the last LAG blocks of this stage's first K word, read at the end of the step before
 #pragma unroll
         for (int i = 0; i < NL; i++) {
+            if (i < LAG && s > 0) unpack(0, NL - LAG + i);
             unpack(1, i);
             mfma2(0, i);
             __builtin_amdgcn_sched_barrier(0);
@@ -559,20 +567,13 @@ __global__ __launch_bounds__(256) void k_mfma_p4(const uint4* __restrict__ Pc, c
         __syncthreads();
         const bool do_ld = FULL || s + 1 < nstep;
         const uint32_t dst = lds0 + (uint32_t)(s % kNS) * (kFR * 1024) + wave * (kFW * 1024);
-        // second K word: first half of the slots issue the LDS reads of the next stage (two per slot) and its loads,
-        // the second half unpacks the next stage's first K word (two blocks per slot)
+        // second K word: every slot issues one LDS read of the next stage and unpacks the block read LAG slots before;
+        // the first kFW slots also issue the loads of stage s + kNS
 #pragma unroll
         for (int i = 0; i < NL; i++) {
-            if (i < NL / 2) {
-                if (do_ld) {
-                    read_raw((s + 1) % kNS, 2 * i);
-                    read_raw((s + 1) % kNS, 2 * i + 1);
-                }
-                if (FULL && i < kFW) dma16(src[i] + (size_t)(s + kNS) * 64, dst + i * 1024);
-            } else if (do_ld) {
-                unpack(0, 2 * (i - NL / 2));
-                unpack(0, 2 * (i - NL / 2) + 1);
-            }
+            if (do_ld) read_raw((s + 1) % kNS, i);
+            if (FULL && i < kFW) dma16(src[i] + (size_t)(s + kNS) * 64, dst + i * 1024);
+            if (do_ld && i >= LAG) unpack(0, i - LAG);
             mfma2(1, i);
             __builtin_amdgcn_sched_barrier(0);
         }
