@@ -1164,6 +1164,7 @@ hipError_t launch_pack4(bool ternary, const int64_t* d_rows, int rows, int Kw, v
     if (grid.y > 65535) return hipErrorInvalidValue;
     const uint32_t* R = reinterpret_cast<const uint32_t*>(d_rows);
     int* sums = packed4_sums(d_out, rows, Kw);
+    if (grid.x > 0x7fffff00u / 32) return hipErrorInvalidValue;
     const int nsum = (int)grid.x * 32;
     if (zero_sums) hipLaunchKernelGGL(k_zero_i32, dim3((nsum + 255) / 256), dim3(256), 0, st, sums, nsum, nullptr, 0);
     if (ternary) hipLaunchKernelGGL((k_pack4<true>), grid, dim3(256), 0, st, R, rows, Kw / 4, static_cast<uint2*>(d_out), sums);
@@ -1287,7 +1288,9 @@ hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* 
     if (f4 && !f4_whole_call_plain(M, KN)) {   // the fp4 GEMM takes its operands at two bits per lane
         void* Ac = d_scratch;
         void* Bc = static_cast<char*>(d_scratch) + mfma_packed4_bytes(M, Kw);
-        const int na = (int)((M + 31) / 32) * 32, nb = (KN + 31) / 32 * 32;   // one launch zeroes both operands' row sums
+        const int64_t na64 = (M + 31) / 32 * 32, nb64 = ((int64_t)KN + 31) / 32 * 32;
+        if (na64 + nb64 > 0x7fffff00LL) return hipErrorInvalidValue;
+        const int na = (int)na64, nb = (int)nb64;   // one launch zeroes both operands' row sums
         hipLaunchKernelGGL(k_zero_i32, dim3((na + nb + 255) / 256), dim3(256), 0, st, packed4_sums(Ac, M, Kw), na,
                            packed4_sums(Bc, KN, Kw), nb);
         hipError_t e = launch_pack4(a_tern, d_a, (int)M, Kw, Ac, false, st);
