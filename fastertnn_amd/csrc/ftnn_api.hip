@@ -113,6 +113,10 @@ static void keep_heap_once() {
         if (!e || atoi(e) == 0) return true;
         mallopt(M_MMAP_THRESHOLD, 32 << 20);
         mallopt(M_TRIM_THRESHOLD, 512 << 20);
+        if (atoi(e) >= 2) {
+            mallopt(M_MMAP_MAX, 0);                    // no mappings at all: results beyond 32 MiB come from the heap too
+            mallopt(M_TRIM_THRESHOLD, 1 << 30);
+        }
         return true;
     }();
     (void)done;
@@ -380,21 +384,124 @@ static void download(void* host, const void* dev, size_t bytes) {
     hip_or_die(hipStreamSynchronize(host_stream()), "hipStreamSynchronize");
 }
 
+// heap memory for a result of kStageFrom bytes or more, as the caller will free() it
+static void* large_alloc(size_t bytes, bool aligned32) {
+    // A large result is often memory the process has not touched yet (a fresh mapping, or new heap), and the copy
+    // into it then pays a page fault per 4 KiB (25 MB: 2.6 ms on one thread, 1.1 ms on eight).  Its 2 MiB-aligned
+    // interior is therefore marked for transparent huge pages: 13 faults instead of 6300 (0.5 ms on one thread)
+    // where the memory is fresh, nothing where the allocator hands out memory that is mapped already.  Still
+    // plain heap memory that the caller free()s; where huge pages are unavailable the hint is ignored.
+    constexpr size_t kHuge = 2u << 20;
+    void* p = aligned32 ? aligned_alloc(32, (bytes + 31) / 32 * 32) : malloc(bytes);
+    static const bool no_thp = getenv("FTNN_HOST_NO_THP") != nullptr;   // tuning aid
+    if (p && !no_thp) {
+        const uintptr_t lo = (reinterpret_cast<uintptr_t>(p) + kHuge - 1) / kHuge * kHuge;
+        const uintptr_t hi = (reinterpret_cast<uintptr_t>(p) + bytes) / kHuge * kHuge;
+        if (hi > lo) (void)madvise(reinterpret_cast<void*>(lo), hi - lo, MADV_HUGEPAGE);
+    }
+    return p;
+}
+
+// Even with huge pages a fresh result costs the copy the time the kernel needs to zero it: the reference's e2e driver
+// on ResNet-152 spends 27 of its 162 ms per pass there (results of 25 and 100 MB, each a new mapping: the allocator
+// returns blocks of that size to the system at once).  A caller that walks the same layers again and again asks for
+// the same sizes again and again, so from the second request for a size on, a thread of its own allocates the next
+// buffer of that size ahead of time and touches its pages; host_alloc hands that one out if it is ready.  The spare
+// is ordinary malloc memory like any other result.  At most kSpareCap bytes wait as spares; a caller confined to
+// fewer than four cores gets none (the thread would take the time from the caller).
+class SparePool {
+public:
+    static SparePool& get() {
+        static SparePool* pool = new SparePool;   // leaked on purpose, like the copy pool
+        return *pool;
+    }
+    // a ready buffer of exactly this kind, or nullptr
+    void* take(size_t bytes, bool aligned32) {
+        if (!running_) return nullptr;
+        std::lock_guard<std::mutex> lock(m_);
+        for (size_t i = 0; i < ready_.size(); i++)
+            if (ready_[i].bytes == bytes && ready_[i].aligned32 == aligned32) {
+                void* p = ready_[i].p;
+                ready_.erase(ready_.begin() + (long)i);
+                held_ -= bytes;
+                return p;
+            }
+        return nullptr;
+    }
+    // a buffer of this kind was just handed out: prepare the next one if the size has been seen before
+    void handed_out(size_t bytes, bool aligned32) {
+        if (!running_) return;
+        std::lock_guard<std::mutex> lock(m_);
+        bool seen = false;
+        for (const Key& k : seen_) seen = seen || (k.bytes == bytes && k.aligned32 == aligned32);
+        if (!seen) {
+            if (seen_.size() < 64) seen_.push_back(Key{bytes, aligned32});
+            return;
+        }
+        for (const Spare& r : ready_)
+            if (r.bytes == bytes && r.aligned32 == aligned32) return;
+        for (const Key& k : wanted_)
+            if (k.bytes == bytes && k.aligned32 == aligned32) return;
+        if (held_ + queued_ + bytes > kSpareCap) return;
+        wanted_.push_back(Key{bytes, aligned32});
+        queued_ += bytes;
+        wake_.notify_one();
+    }
+
+private:
+    static constexpr size_t kSpareCap = 512u << 20;
+    struct Key {
+        size_t bytes;
+        bool aligned32;
+    };
+    struct Spare {
+        void* p;
+        size_t bytes;
+        bool aligned32;
+    };
+    SparePool() {
+        cpu_set_t set;
+        int cores = 1;
+        if (sched_getaffinity(0, sizeof(set), &set) == 0) cores = CPU_COUNT(&set);
+        if (cores < 4 || getenv("FTNN_HOST_NO_SPARES")) return;   // (the variable: tuning aid)
+        try {
+            std::thread([this] { run(); }).detach();
+            running_ = true;
+        } catch (const std::system_error&) {
+        }
+    }
+    void run() {
+        for (;;) {
+            std::unique_lock<std::mutex> lock(m_);
+            wake_.wait(lock, [this] { return !wanted_.empty(); });
+            const Key k = wanted_.front();
+            wanted_.erase(wanted_.begin());
+            lock.unlock();
+            unsigned char* p = static_cast<unsigned char*>(large_alloc(k.bytes, k.aligned32));
+            if (p)
+                for (size_t i = 0; i < k.bytes; i += 4096) p[i] = 0;   // maps the page (a huge page where there is one)
+            lock.lock();
+            queued_ -= k.bytes;
+            if (p) {
+                ready_.push_back(Spare{p, k.bytes, k.aligned32});
+                held_ += k.bytes;
+            }
+        }
+    }
+    std::mutex m_;
+    std::condition_variable wake_;
+    std::vector<Key> seen_, wanted_;
+    std::vector<Spare> ready_;
+    size_t held_ = 0, queued_ = 0;
+    bool running_ = false;
+};
+
 static void* host_alloc(size_t bytes, bool aligned32) {
     void* p;
-    constexpr size_t kHuge = 2u << 20;
     if (bytes >= kStageFrom) {
-        // A large result is often memory the process has not touched yet (a fresh mapping, or new heap), and the copy
-        // into it then pays a page fault per 4 KiB (25 MB: 2.6 ms on one thread, 1.1 ms on eight).  Its 2 MiB-aligned
-        // interior is therefore marked for transparent huge pages: 13 faults instead of 6300 (0.5 ms on one thread)
-        // where the memory is fresh, nothing where the allocator hands out memory that is mapped already.  Still
-        // plain heap memory that the caller free()s; where huge pages are unavailable the hint is ignored.
-        p = aligned32 ? aligned_alloc(32, (bytes + 31) / 32 * 32) : malloc(bytes);
-        if (p) {
-            const uintptr_t lo = (reinterpret_cast<uintptr_t>(p) + kHuge - 1) / kHuge * kHuge;
-            const uintptr_t hi = (reinterpret_cast<uintptr_t>(p) + bytes) / kHuge * kHuge;
-            if (hi > lo) (void)madvise(reinterpret_cast<void*>(lo), hi - lo, MADV_HUGEPAGE);
-        }
+        p = SparePool::get().take(bytes, aligned32);
+        if (!p) p = large_alloc(bytes, aligned32);
+        if (p) SparePool::get().handed_out(bytes, aligned32);
     } else if (aligned32) {
         // aligned_alloc(32, ...) as src/tnns/ternarize2row_avx2.c:735
         p = aligned_alloc(32, (bytes + 31) / 32 * 32);
@@ -1153,7 +1260,7 @@ void tnns_conv(testcase_t* t) {
         return ts.tv_sec * 1e6 + ts.tv_nsec * 1e-3;
     };
     const double T0 = nowus();
-    float* y = (float*)host_alloc(y_bytes, false);   // before the device work: its pages can be mapped meanwhile
+    float* y = (float*)host_alloc(y_bytes, false);
     const double T1 = nowus();
     float* d_x = (float*)upload(SLOT_X, t->input, (size_t)N * C * H * W * sizeof(float));
     float* d_thr = (float*)upload(SLOT_THR, t->input_thresholds, (size_t)N * sizeof(float));
