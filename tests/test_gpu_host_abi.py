@@ -101,6 +101,39 @@ def test_large_buffers_through_the_host_entry_points(hip, oracle):
     assert y_h.tobytes() == want.tobytes()
 
 
+def test_results_prepared_ahead_of_time(hip, oracle):
+    """From the second request for a size on, large results come from buffers a helper thread allocated and touched
+    beforehand: a run of calls with two alternating result sizes, some results held while later ones are made, every
+    one complete, distinct and the caller's to free."""
+    import ctypes
+    la = make_layer(TNN, (16, 64, 64, 40, 3, 3, 1, 1), 8, seed=77)     # 5.2 MB result
+    lb = make_layer(TNN, (16, 64, 64, 72, 1, 1, 0, 1), 8, seed=78)     # 9.4 MB result
+    cases = []
+    for L in (la, lb):
+        qw = oracle.pack_weights(L["w"], L["wthr"], True)
+        want = oracle.conv(TNN, L["x"], L["thr"], qw, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], L["alpha"])
+        assert want.nbytes >= 4 << 20
+        cases.append((L, qw, want))
+    held = []
+    for rep in range(10):
+        L, qw, want = cases[rep % 2]
+        x, thr = np.ascontiguousarray(L["x"]), np.ascontiguousarray(L["thr"])
+        t = hip.Testcase(type=TNN, batchcount=8, channelcount=L["c"], inputW=L["iw"], inputH=L["ih"], kernelcount=L["kn"],
+                         kernelW=L["kw"], kernelH=L["kh"], paddingW=L["pad"], paddingH=L["pad"], strideW=L["stride"],
+                         strideH=L["stride"], preluAlpha=L["alpha"], input_thresholds=thr.ctypes.data, input=x.ctypes.data,
+                         quantized_kernel_packing2=qw.ctypes.data)
+        print("case prepared results", rep, flush=True)
+        hip._L.tnns_conv(ctypes.byref(t))
+        got = np.ctypeslib.as_array(ctypes.cast(t.output, ctypes.POINTER(ctypes.c_float)), shape=(want.size,))
+        assert got.tobytes() == want.tobytes(), rep
+        held.append(t.output)
+        if len(held) > 3:                      # the caller frees in its own order, three results later
+            hip._libc.free(ctypes.c_void_p(held.pop(0)))
+    assert len(set(held)) == len(held)
+    for p in held:
+        hip._libc.free(ctypes.c_void_p(p))
+
+
 _CHILD = r"""
 import sys
 import numpy as np, torch
