@@ -135,18 +135,27 @@ def graph_times(torch, fn, y, reps, n_graph=10):
     fn()
     torch.cuda.synchronize()
     y_eager = y.clone()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        for _ in range(n_graph):
-            fn()
-    y.zero_()
-    graph.replay()
-    torch.cuda.synchronize()
-    same = bool(torch.equal(y, y_eager))
-    ms = sorted(event_times(torch, graph.replay, reps))[reps // 2] / n_graph
-    same = same and bool(torch.equal(y, y_eager))
-    del graph
-    return ms, same
+    try:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(n_graph):
+                fn()
+        y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        same = bool(torch.equal(y, y_eager))
+        ms = sorted(event_times(torch, graph.replay, reps))[reps // 2] / n_graph
+        same = same and bool(torch.equal(y, y_eager))
+        del graph
+        return ms, same
+    except RuntimeError as e:      # no graph on this runtime: eager calls back to back instead, and say so
+        sys.stderr.write("bench.py: graph capture failed (%s); timing %d eager calls back to back\n" % (e, n_graph))
+        torch.cuda.synchronize()
+
+        def many():
+            for _ in range(n_graph):
+                fn()
+        return sorted(event_times(torch, many, reps))[reps // 2] / n_graph, None
 
 
 def small_gemm(torch, lib, m, n, k, reps=30):
