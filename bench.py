@@ -378,6 +378,13 @@ def e2e_latency(torch, lib, batch, reps=50, cpu=True, typ=None):
                 net.run(x, out=y, graph=graph)
             t = sorted(event_times(torch, lambda: net.run(x, out=y, graph=graph), reps))[reps // 2]
             out[key] = round(t, 4)
+
+            # ten passes queued behind each other: the device's time per pass without the host's part in a single call
+            def ten(graph=graph):
+                for _ in range(10):
+                    net.run(x, out=y, graph=graph)
+            t10 = sorted(event_times(torch, ten, max(5, reps // 2)))[max(5, reps // 2) // 2] / 10
+            out[key.replace("_ms", "_ms_per_pass_of_ten_queued")] = round(t10, 4)
     st.synchronize()
     from oracle import ftnn_oracle as O
     if cpu and O.Reference.available():
