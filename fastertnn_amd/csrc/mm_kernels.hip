@@ -105,8 +105,13 @@ __device__ __forceinline__ uint32_t popc4(const uint4& v) {
 // im2row matrix is never written to memory.
 // TR = true stores the result transposed, Y[column * M + row] (row-major GEMM results only): the
 // launcher uses it to run a BTN GEMM as a TBN GEMM with the operands exchanged, see launch_mm.
-template <int MODE, int TM, int TN, int GC, bool IMPL, bool TR = false>
-__global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
+// KS = 4 or 8 splits K over the KS wavefronts of a workgroup, for problems whose tiles alone leave most of the chip
+// idle (the reference's CPU-sized GEMM, 256 x 256 x 4096, is 128 workgroups of the smallest tile on 256 compute
+// units): a chunk is GC = KS groups, wavefront w takes group w of every chunk for all TN columns of the workgroup
+// (four times the workgroups of KS / 4 times the wavefronts, 1 / KS of the K loop each), and the partial counts meet
+// in LDS at the end, where wavefront 0 finishes the tile.  Integer counts: any order of the sum is exact.
+template <int MODE, int TM, int TN, int GC, bool IMPL, bool TR = false, int KS = 0>
+__global__ __launch_bounds__(KS ? 64 * KS : 256) void k_mm(const uint32_t* __restrict__ A,
                                             const uint32_t* __restrict__ B,
                                             float* __restrict__ Y, int M, int KN, int OHW, int G,
                                             int K_unpack, float alpha, FastDiv dOHW, ConvGeom cg, QuantOut qo,
@@ -117,9 +122,14 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
     constexpr int LDW = GC * AG + 4;           // LDS row stride in dwords (padded)
     constexpr int QPR = GC * AG / 4;           // 16-byte quads per row and chunk
     constexpr int QUADS = BM * QPR;            // quads per chunk
-    constexpr int IT = (QUADS + 255) / 256;    // staging passes per thread
-    constexpr int RPI = 256 / QPR;             // rows covered by one staging pass
-    static_assert(256 % QPR == 0, "a staging pass must cover whole rows");
+    constexpr int NW = KS ? KS : 4, NT = 64 * NW;   // wavefronts and threads of a workgroup
+    constexpr int IT = (QUADS + NT - 1) / NT;  // staging passes per thread
+    constexpr int RPI = NT / QPR;              // rows covered by one staging pass
+    static_assert(NT % QPR == 0, "a staging pass must cover whole rows");
+    static_assert(!KS || (GC == KS && !IMPL), "the K split hands one group of a chunk to each wavefront");
+    // counts a wavefront hands over under the K split: cn, and what the type has of cz, rowz, colz
+    constexpr int NV = TM * TN * (MODE == kTNN ? 2 : 1) + (MODE == kTBN ? TM : 0) + (MODE == kBTN ? TN : 0);
+    static_assert(!KS || (NW - 1) * NV * 64 <= 2 * BM * LDW, "the partial counts fit the operand buffers");
     __shared__ uint32_t lds[2][BM * LDW];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -138,7 +148,7 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
         bx = p * (uint32_t)panel + (within - by * pw);
     }
     const int64_t row0 = (int64_t)bx * BM;
-    const int col0 = (by * 4 + wave) * TN;
+    const int col0 = KS ? (int)by * TN : (int)(by * 4 + wave) * TN;
     const size_t RDA = (size_t)G * AG, RDB = (size_t)G * BG;
 
     uint32_t cn[TM][TN];  // popcount of "negative product" lanes
@@ -164,7 +174,7 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
 
     // staging map (explicit rows): pass `it` of this thread moves quad sq of tile row sr + it*RPI
     const int sq = IMPL ? (tid & 3) : tid % QPR, sr = IMPL ? (tid >> 2) : tid / QPR;
-    const bool stager = IMPL || (QUADS % 256 == 0) || (tid < QUADS);
+    const bool stager = IMPL || (QUADS % NT == 0) || (tid < QUADS);
     const uint32_t* ap[IT];
     uint32_t* const lw = &lds[0][0] + sr * LDW + sq * (IMPL ? 2 : 4);
     uint4 stage[IT];
@@ -260,7 +270,8 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
         const bool more = c + 1 < nchunk;
         if (more) fetch(g0 + GC);  // the loads of the next chunk land after the arithmetic
         const uint32_t* lr = &lds[c & 1][0];
-        for (int g = 0; g < gc; g++) {
+        // K split: this wavefront's group of the chunk, if the chunk has it (only the last chunk can be short)
+        for (int g = KS ? wave : 0; g < (KS ? min(gc, wave + 1) : gc); g++) {
             uint4 sa0[TM], sa1[TM], za0[TM], za1[TM];
 #pragma unroll
             for (int a = 0; a < TM; a++) {
@@ -307,6 +318,33 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
         __syncthreads();
     }
 
+    if constexpr (KS) {
+        // the loop's last barrier has passed: the operand buffers are free for the partial counts [wavefront - 1][count][lane]
+        uint32_t* red = &lds[0][0];
+        auto each = [&](auto&& fn) {
+            int v = 0;
+#pragma unroll
+            for (int a = 0; a < TM; a++)
+#pragma unroll
+                for (int b = 0; b < TN; b++) {
+                    fn(cn[a][b], v++);
+                    if (MODE == kTNN) fn(cz[a][b], v++);
+                }
+            if (MODE == kTBN) {
+#pragma unroll
+                for (int a = 0; a < TM; a++) fn(rowz[a], v++);
+            }
+            if (MODE == kBTN) {
+#pragma unroll
+                for (int b = 0; b < TN; b++) fn(colz[b], v++);
+            }
+        };
+        if (wave != 0) each([&](uint32_t& c, int v) { red[((wave - 1) * NV + v) * 64 + lane] = c; });
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int w = 0; w < NW - 1; w++) each([&](uint32_t& c, int v) { c += red[(w * NV + v) * 64 + lane]; });
+    }
     const int lanes_total = G * 4 * 64;  // 64 * Kw
     // PReLU in the reference's form for the type, from the integer accumulators of (row a, column b)
     auto finish = [&](int a, int b) -> float {
@@ -377,17 +415,18 @@ __global__ __launch_bounds__(256) void k_mm(const uint32_t* __restrict__ A,
     }
 }
 
-template <int MODE, int TM, int TN, int GC, bool IMPL, bool TR>
+template <int MODE, int TM, int TN, int GC, bool IMPL, bool TR, int KS = 0>
 hipError_t launch_cfg(const uint32_t* A, const uint32_t* B, float* Y, int64_t M, int KN, int OHW,
                       int G, int K_unpack, float alpha, const ConvGeom& cg, hipStream_t st, const QuantOut& qo) {
     const int64_t gx = (M + 64 * TM - 1) / (64 * TM);
     // with a quantised hand-over every 64-channel word that holds a kernel is written in full
     const int cols = qo.mode != 0 ? (KN + 63) / 64 * 64 : KN;
-    const int64_t gy = (cols + 4 * TN - 1) / (4 * TN);
+    constexpr int WC = KS ? TN : 4 * TN;   // columns of a workgroup
+    const int64_t gy = (cols + WC - 1) / WC;
     if (gx > 0x7fffffffLL || gy > 65535) return hipErrorInvalidValue;
     static const int tune_panel = getenv("FTNN_MM_PANEL") ? atoi(getenv("FTNN_MM_PANEL")) : 32;   // tuning aid
     const int panel = (gx >= 32 && gy >= 32 && gx * gy < 0x7fffffffLL) ? tune_panel : 0;
-    hipLaunchKernelGGL((k_mm<MODE, TM, TN, GC, IMPL, TR>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
+    hipLaunchKernelGGL((k_mm<MODE, TM, TN, GC, IMPL, TR, KS>), dim3((unsigned)gx, (unsigned)gy), dim3(KS ? 64 * KS : 256), 0, st,
                        A, B, Y, (int)M, KN, OHW, G, K_unpack, alpha, make_fastdiv((uint32_t)OHW), cg, qo, panel);
     return hipGetLastError();
 }
@@ -410,6 +449,23 @@ hipError_t launch_mode(const uint32_t* A, const uint32_t* B, float* Y, int64_t M
     if (tm == TM_ && tn == TN_) return launch_cfg<MODE, TM_, TN_, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
         FTNN_TRY(2, 8) FTNN_TRY(1, 8) FTNN_TRY(1, 4) FTNN_TRY(1, 2)
 #undef FTNN_TRY
+    }
+    // Few tiles and a K loop worth splitting: the wavefronts of a workgroup share K (KS in the kernel).  Measured on
+    // MI355X as device time per call with ten calls queued behind each other: 256 x 256 x 4096 8.7 -> 5.4 us (3.2 us is
+    // what the smallest problem takes, 1.7 us the vector ALU's own time for this one), 128 x 1024 x 2048 5.6 -> 5.1,
+    // 1024 x 128 x 8192 14 -> 9.5; from 512 x 512 x 4096 on the plain tiles are as fast.  FTNN_MM_KSPLIT = 0 switches
+    // it off, "W,TN" forces W = 4 or 8 wavefronts on TN = 2 or 4 columns (tuning aid).
+    if constexpr (!IMPL) {
+        static const char* tune_ks = getenv("FTNN_MM_KSPLIT");
+        int w = 0, tn = 0;
+        if (tune_ks) sscanf(tune_ks, "%d,%d", &w, &tn);
+        else if (!force && wgs(1, 2) <= 256 && G >= 4) w = G >= 8 ? 8 : 4, tn = ((M + 63) / 64) * ((KN + 3) / 4) < 256 ? 2 : 4;
+        if (w && qo.mode == 0) {
+#define FTNN_TRY(W_, TN_) \
+    if (w == W_ && tn == TN_) return launch_cfg<MODE, 1, TN_, W_, false, TR, W_>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
+            FTNN_TRY(4, 2) FTNN_TRY(4, 4) FTNN_TRY(8, 2) FTNN_TRY(8, 4)
+#undef FTNN_TRY
+        }
     }
     if (wgs(2, 8) >= 3072) return launch_cfg<MODE, 2, 8, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);
     if (wgs(1, 8) >= 1536) return launch_cfg<MODE, 1, 8, 1, IMPL, TR>(A, B, Y, M, KN, OHW, G, K_unpack, alpha, cg, st, qo);

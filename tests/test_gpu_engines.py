@@ -166,6 +166,68 @@ def test_vector_alu_gemm_walks_large_grids_in_panels(hip, oracle, typ, shape):
     assert y.cpu().numpy().tobytes() == want.tobytes()
 
 
+# shapes (n, oh, ow, kn, words) that the vector-ALU GEMM runs with K split over the wavefronts of a workgroup: few tiles,
+# rows of 16 words and more.  By the launcher's rule these take 4 wavefronts x 2 columns, 8 x 4, 8 x 2 (K tail: 25
+# groups in chunks of 8), 4 x 4, and conv-shaped results with 4 and 8 wavefronts.
+KSPLIT_SHAPES = [(70, 1, 1, 100, 16), (256, 1, 1, 256, 64), (90, 1, 1, 70, 100), (64, 1, 1, 2048, 20), (2, 7, 9, 50, 24),
+                 (3, 5, 5, 40, 36), (1, 1, 1, 64, 16), (64, 1, 1, 3, 44)]
+
+
+def _ksplit_case(hip, oracle, typ, shape, alpha=0.5):
+    import torch
+    n, oh, ow, kn, kw = shape
+    m = n * oh * ow
+    rng = np.random.default_rng(1000 * typ + m + kn + kw)
+    at, wt = act_is_ternary(typ), weight_is_ternary(typ)
+    a = rng.integers(-2 ** 63, 2 ** 63, size=m * kw * (2 if at else 1), dtype=np.int64)
+    b = rng.integers(-2 ** 63, 2 ** 63, size=kn * kw * (2 if wt else 1), dtype=np.int64)
+    ku = 64 * kw - 7
+    want = oracle.mm(typ, a, b, n, oh, ow, kn, kw, alpha, ku)
+    y = torch.full((n, kn, oh, ow), float("nan"), dtype=torch.float32, device="cuda")
+    hip.mm_engine(hip.ENGINE_VALU, typ, _dev(a), _dev(b), n, oh, ow, kn, kw, alpha, ku, out=y)
+    assert y.cpu().numpy().tobytes() == want.tobytes(), (typ, shape, alpha)
+
+
+@pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
+@pytest.mark.parametrize("shape", KSPLIT_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_vector_alu_gemm_splits_k_for_small_problems(hip, oracle, typ, shape):
+    """small GEMMs (the reference's CPU-sized case among them) run with the wavefronts of a workgroup sharing K and
+    their partial counts summed through LDS: every type, row-major and NCHW results, ragged rows and columns, K tails
+    that leave wavefronts without a group, both slopes"""
+    print("case", TYPE_NAMES[typ], shape, flush=True)
+    for alpha in (0.5, -0.25):
+        _ksplit_case(hip, oracle, typ, shape, alpha)
+
+
+_KSPLIT_CHILD = r"""
+import sys
+sys.path.insert(0, sys.argv[1])
+import fastertnn_amd.lib as hip
+from oracle.ftnn_oracle import Oracle
+from tests.test_gpu_engines import KSPLIT_SHAPES, _ksplit_case
+oracle = Oracle()
+for typ in range(4):
+    for shape in KSPLIT_SHAPES:
+        print("case", typ, shape, flush=True)
+        _ksplit_case(hip, oracle, typ, shape)
+print("child ok")
+"""
+
+
+@pytest.mark.parametrize("variant", ["4,2", "4,4", "8,2", "8,4", "0"])
+def test_every_k_split_variant_forced(variant):
+    """FTNN_MM_KSPLIT forces each split variant (wavefronts, columns) onto every shape above, whatever the launcher's
+    own rule would pick, and switches the split off; the switch is read once per process, hence child processes"""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    print("case forced K split", variant, flush=True)
+    r = subprocess.run([sys.executable, "-c", _KSPLIT_CHILD, root], env=dict(os.environ, FTNN_MM_KSPLIT=variant),
+                       capture_output=True, text=True, timeout=280)
+    assert r.returncode == 0 and "child ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+
+
 def test_lanes_flagged_zero_and_negative_count_as_zero(hip, oracle):
     """a lane with both its sign and its zero bit set is zero in the reference's formula
     (za|zb masks it); the expanded operands must agree"""
