@@ -6,7 +6,8 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libftnn_hip.so")
-SOURCES = ["ftnn_api.hip", "pack_kernels.hip", "mm_kernels.hip", "mfma_kernels.hip", "stem_kernels.hip", "ftnn_net.hip"]
+SOURCES = ["ftnn_api.hip", "pack_kernels.hip", "mm_kernels.hip", "mfma_kernels.hip", "stem_kernels.hip", "ftnn_net.hip",
+           "host_hash.cpp"]   # the last one is plain host C++
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -44,9 +45,11 @@ def build_library(verbose=False):
     objs = []
     procs = []
     for src in SOURCES:
-        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+        obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
         objs.append(obj)
         cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+        if src.endswith(".cpp"):
+            cmd = [HIPCC, "-x", "c++", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-c", os.path.join(CSRC, src), "-o", obj]
         if src in NO_SCRATCH:
             cmd.append("-Rpass-analysis=kernel-resource-usage")
         if verbose:

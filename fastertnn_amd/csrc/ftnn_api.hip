@@ -12,6 +12,7 @@
 
 #include <algorithm>
 #include <condition_variable>
+#include <functional>
 #include <mutex>
 #include <system_error>
 #include <thread>
@@ -19,6 +20,7 @@
 
 #include "../../include/ftnn.h"
 #include "ftnn_internal.h"
+#include "host_hash.h"
 
 namespace ftnn {
 
@@ -76,10 +78,12 @@ int check_conv_shape(int N, int C, int H, int W, int H_pad, int W_pad, int kH, i
 }
 
 // ---- lazily created state behind the host-memory entry points ----
+// grow-only device buffers of the host entry points, one per kind of operand
+enum { SLOT_X = 0, SLOT_THR, SLOT_W, SLOT_ROWS, SLOT_SCRATCH, SLOT_Y, SLOT_PREP, SLOT_COUNT };
 struct HostCtx {
     hipStream_t stream = nullptr;
-    void* buf[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
-    size_t cap[6] = {0, 0, 0, 0, 0, 0};
+    void* buf[SLOT_COUNT] = {};
+    size_t cap[SLOT_COUNT] = {};
 };
 static HostCtx g_ctx;
 // The reference's entry points are called from one thread (its drivers are single-threaded); the
@@ -157,8 +161,9 @@ constexpr size_t kStageChunk = 4u << 20;   // bytes per chunk (2, 8 and 16 MiB m
 constexpr int kStageSlots = 4;
 constexpr size_t kStageFrom = 4u << 20;    // smaller copies take the plain path (the ring's event waits cost more)
 
-// A fixed set of worker threads that copy slices of one memcpy; created on first use and never joined (the object
-// is leaked on purpose: at exit the workers are blocked on its condition variable).
+// A fixed set of worker threads that work on page-aligned slices of one buffer -- slices of one memcpy, or of one
+// content hash; created on first use and never joined (the object is leaked on purpose: at exit the workers are blocked
+// on its condition variable).
 class CopyPool {
 public:
     static CopyPool& get() {
@@ -167,14 +172,17 @@ public:
     }
     // with one thread the runtime's own pageable copy is the faster one (29 GB/s up against a single memcpy into the ring)
     bool parallel() const { return workers_ > 0; }
-    void copy(void* dst, const void* src, size_t bytes) {
-        if (workers_ == 0 || bytes < (256u << 10)) {
-            memcpy(dst, src, bytes);
+    // slices a job is cut into: one per worker and one for the caller
+    int parts() const { return workers_ + 1; }
+    typedef std::function<void(int part, size_t lo, size_t hi)> Job;
+    // fn(part, lo, hi) for every slice [lo, hi) of [0, bytes), each on a thread of its own; returns when all are done
+    void run_slices(size_t bytes, const Job& fn) {
+        if (workers_ == 0) {
+            fn(0, 0, bytes);
             return;
         }
         std::unique_lock<std::mutex> lock(m_);
-        dst_ = static_cast<char*>(dst);
-        src_ = static_cast<const char*>(src);
+        job_ = &fn;
         bytes_ = bytes;
         pending_ = workers_;
         generation_++;
@@ -183,6 +191,15 @@ public:
         slice(workers_);   // the calling thread takes the last slice
         lock.lock();
         done_.wait(lock, [this] { return pending_ == 0; });
+    }
+    void copy(void* dst, const void* src, size_t bytes) {
+        if (workers_ == 0 || bytes < (256u << 10)) {
+            memcpy(dst, src, bytes);
+            return;
+        }
+        char* d = static_cast<char*>(dst);
+        const char* s = static_cast<const char*>(src);
+        run_slices(bytes, [d, s](int, size_t lo, size_t hi) { memcpy(d + lo, s + lo, hi - lo); });
     }
 
 private:
@@ -209,7 +226,7 @@ private:
         const size_t per = (bytes_ / parts + 4095) & ~(size_t)4095;   // whole pages per thread
         const size_t lo = std::min(bytes_, per * (size_t)t), hi = std::min(bytes_, lo + per);
         const size_t end = t == workers_ ? bytes_ : hi;
-        if (end > lo) memcpy(dst_ + lo, src_ + lo, end - lo);
+        (*job_)(t, lo, std::max(lo, end));   // an empty slice is still reported: a job may keep a result per part
     }
     void run(int t) {
         uint64_t seen = 0;
@@ -225,8 +242,7 @@ private:
     }
     std::mutex m_;
     std::condition_variable wake_, done_;
-    char* dst_ = nullptr;
-    const char* src_ = nullptr;
+    const Job* job_ = nullptr;
     size_t bytes_ = 0;
     int workers_ = 0, pending_ = 0;
     uint64_t generation_ = 0;
@@ -415,6 +431,15 @@ public:
         static SparePool* pool = new SparePool;   // leaked on purpose, like the copy pool
         return *pool;
     }
+    // frees every spare that is ready (those being prepared arrive later and age out)
+    void release() {
+        if (!running_) return;
+        std::lock_guard<std::mutex> lock(m_);
+        for (const Spare& r : ready_) free(r.p);
+        ready_.clear();
+        held_ = 0;
+        seen_.clear();
+    }
     // a ready buffer of exactly this kind, or nullptr
     void* take(size_t bytes, bool aligned32) {
         if (!running_) return nullptr;
@@ -432,6 +457,17 @@ public:
     void handed_out(size_t bytes, bool aligned32) {
         if (!running_) return;
         std::lock_guard<std::mutex> lock(m_);
+        // a spare that kSpareMaxAge large results have passed by belongs to a caller that has moved on: free it
+        clock_++;
+        for (size_t i = 0; i < ready_.size();) {
+            if (clock_ - ready_[i].born > kSpareMaxAge) {
+                free(ready_[i].p);
+                held_ -= ready_[i].bytes;
+                ready_.erase(ready_.begin() + (long)i);
+            } else {
+                i++;
+            }
+        }
         bool seen = false;
         for (const Key& k : seen_) seen = seen || (k.bytes == bytes && k.aligned32 == aligned32);
         if (!seen) {
@@ -450,6 +486,7 @@ public:
 
 private:
     static constexpr size_t kSpareCap = 512u << 20;
+    static constexpr uint64_t kSpareMaxAge = 256;
     struct Key {
         size_t bytes;
         bool aligned32;
@@ -458,6 +495,7 @@ private:
         void* p;
         size_t bytes;
         bool aligned32;
+        uint64_t born;   // clock_ when it became ready
     };
     SparePool() {
         cpu_set_t set;
@@ -483,7 +521,7 @@ private:
             lock.lock();
             queued_ -= k.bytes;
             if (p) {
-                ready_.push_back(Spare{p, k.bytes, k.aligned32});
+                ready_.push_back(Spare{p, k.bytes, k.aligned32, clock_});
                 held_ += k.bytes;
             }
         }
@@ -493,6 +531,7 @@ private:
     std::vector<Key> seen_, wanted_;
     std::vector<Spare> ready_;
     size_t held_ = 0, queued_ = 0;
+    uint64_t clock_ = 0;
     bool running_ = false;
 };
 
@@ -515,8 +554,6 @@ static void* host_alloc(size_t bytes, bool aligned32) {
     return p;
 }
 
-enum { SLOT_X = 0, SLOT_THR, SLOT_W, SLOT_ROWS, SLOT_SCRATCH, SLOT_Y };
-
 // the pinned area an operand below kStageFrom is staged through: the activation-side operand, the weight-side
 // operand and the thresholds of one call each have their own
 static int area_of_slot(int slot) {
@@ -533,14 +570,18 @@ static int area_of_slot(int slot) {
 // The reference's layer functions read the packed weights where they lie; here they must reach the device and, for
 // the matrix-core engine, be re-arranged into fragments: an upload, a launch and their latencies on every call for
 // data that a network never changes.  tnns_conv therefore keeps the prepared weights of the layers it has seen,
-// found again by host address, size, layer shape and a 64-bit hash of the CONTENTS, which is recomputed on every
-// call: a caller that frees the rows and packs another layer's at the same address, or rewrites them in place,
-// gets a different hash and a fresh upload.  Entries are dropped least recently used first beyond 512 entries or
-// 1 GiB of device memory.
+// found again by byte count, layer shape and a 128-bit hash of the CONTENTS, recomputed on every call: rows that are
+// rewritten in place, or another layer's rows packed into memory that malloc hands out again, give another hash and
+// a fresh upload; the same rows packed again at another address are found.  The host address is not part of the
+// identity.  The hash must cost less than the upload it saves: it runs on AES rounds where the CPU has them (limited
+// by memory bandwidth), rows of 1 MiB and more are hashed in slices on the copy threads, and rows beyond
+// kWeightCacheMaxRows bytes are not kept at all but uploaded and prepared on every call, which at that size costs no
+// more than reading them once on the host.  Entries are dropped least recently used first beyond 512 entries or the
+// byte cap (1 GiB of device memory; FTNN_HOST_WEIGHT_CACHE_MB = n sets it, FTNN_HOST_NO_WEIGHT_CACHE = 1 or a cap of 0
+// switches the cache off); ftnn_host_forget_weights() drops them all.
 struct PreparedWeights {
-    const void* host;
     size_t bytes;
-    uint64_t hash;
+    Hash128 hash;
     int type, C, KN, KH, KW;
     void* dev;
     size_t dev_bytes;
@@ -549,50 +590,62 @@ struct PreparedWeights {
 static std::vector<PreparedWeights> g_weights;
 static uint64_t g_weights_clock = 0;
 static size_t g_weights_bytes = 0;
-constexpr size_t kWeightCacheEntries = 512, kWeightCacheBytes = (size_t)1 << 30;
+constexpr size_t kWeightCacheEntries = 512;
+constexpr size_t kWeightCacheMaxRows = (size_t)16 << 20;   // packed rows beyond this are not cached
+constexpr size_t kParallelHashFrom = (size_t)1 << 20;
 
-// 64-bit hash of `bytes` (a multiple of 32: packed rows are whole groups of 4 words): four independent
-// multiply-rotate lanes over 32-byte blocks, folded at the end
-static uint64_t content_hash(const void* data, size_t bytes) {
-    const uint64_t* p = static_cast<const uint64_t*>(data);
-    uint64_t h0 = 0x9E3779B97F4A7C15ull, h1 = 0xC2B2AE3D27D4EB4Full, h2 = 0x165667B19E3779F9ull, h3 = 0x27D4EB2F165667C5ull;
-    auto rotl = [](uint64_t v, int r) { return (v << r) | (v >> (64 - r)); };
-    const size_t blocks = bytes / 32;
-    for (size_t i = 0; i < blocks; i++, p += 4) {
-        h0 = rotl((h0 ^ p[0]) * 0xFF51AFD7ED558CCDull, 29);
-        h1 = rotl((h1 ^ p[1]) * 0xC4CEB9FE1A85EC53ull, 31);
-        h2 = rotl((h2 ^ p[2]) * 0x9FB21C651E98DF25ull, 27);
-        h3 = rotl((h3 ^ p[3]) * 0xD6E8FEB86659FD93ull, 33);
-    }
-    const unsigned char* tail = reinterpret_cast<const unsigned char*>(p);
-    for (size_t i = 0; i < bytes % 32; i++) h0 = rotl((h0 ^ tail[i]) * 0xFF51AFD7ED558CCDull, 29);
-    uint64_t h = h0 ^ rotl(h1, 17) ^ rotl(h2, 34) ^ rotl(h3, 51) ^ (uint64_t)bytes;
-    h ^= h >> 33;
-    h *= 0xFF51AFD7ED558CCDull;
-    h ^= h >> 29;
-    return h;
+static size_t weight_cache_cap() {
+    static const size_t cap = []() -> size_t {
+        if (const char* off = getenv("FTNN_HOST_NO_WEIGHT_CACHE"))
+            if (atoi(off) != 0) return 0;
+        if (const char* mb = getenv("FTNN_HOST_WEIGHT_CACHE_MB")) return (size_t)std::max(0LL, atoll(mb)) << 20;
+        return (size_t)1 << 30;
+    }();
+    return cap;
+}
+
+// 128-bit hash of the packed rows; from kParallelHashFrom bytes on, the slices of the copy threads are hashed side by
+// side and their hashes hashed in order (the number of slices is fixed per process, so the result is stable)
+static Hash128 content_hash(const void* data, size_t bytes) {
+    CopyPool& pool = CopyPool::get();
+    if (bytes < kParallelHashFrom || !pool.parallel()) return hash128(data, bytes, 0);
+    Hash128 part[32] = {};
+    const char* base = static_cast<const char*>(data);
+    pool.run_slices(bytes, [&part, base](int t, size_t lo, size_t hi) { part[t & 31] = hash128(base + lo, hi - lo, (uint64_t)t + 1); });
+    return hash128(part, sizeof(Hash128) * (size_t)std::min(pool.parts(), 32), bytes);
+}
+
+static void drop_weight_entry(size_t i) {
+    hip_or_die(hipStreamSynchronize(host_stream()), "hipStreamSynchronize");
+    hip_or_die(hipFree(g_weights[i].dev), "hipFree");
+    g_weights_bytes -= g_weights[i].dev_bytes;
+    g_weights.erase(g_weights.begin() + (long)i);
 }
 
 // device pointer of the prepared weights of this layer (uploading and preparing them on a miss)
 static const void* prepared_weights(int type, const int64_t* host, size_t bytes, int C, int KN, int KH, int KW) {
-    const uint64_t hash = content_hash(host, bytes);
+    const size_t dev_bytes = (size_t)ftnn_conv_weights_bytes(type, C, KN, KH, KW);
+    const size_t cap = weight_cache_cap();
+    if (cap == 0 || bytes > kWeightCacheMaxRows || dev_bytes > cap) {
+        // not kept: uploaded and prepared into a work buffer on every call
+        void* d_prep = dev_buf(SLOT_PREP, dev_bytes);
+        int64_t* d_rows = (int64_t*)upload(SLOT_W, host, bytes);
+        if (ftnn_conv_prepare_weights(type, d_rows, C, KN, KH, KW, d_prep, host_stream()) != FTNN_OK) die("tnns_conv");
+        return d_prep;
+    }
+    const Hash128 hash = content_hash(host, bytes);
     g_weights_clock++;
     for (PreparedWeights& e : g_weights)
-        if (e.host == host && e.bytes == bytes && e.hash == hash && e.type == type && e.C == C && e.KN == KN && e.KH == KH &&
-            e.KW == KW) {
+        if (e.bytes == bytes && e.hash == hash && e.type == type && e.C == C && e.KN == KN && e.KH == KH && e.KW == KW) {
             e.last_use = g_weights_clock;
             return e.dev;
         }
-    PreparedWeights e = {host, bytes, hash, type, C, KN, KH, KW, nullptr, (size_t)ftnn_conv_weights_bytes(type, C, KN, KH, KW),
-                         g_weights_clock};
-    while (!g_weights.empty() && (g_weights.size() >= kWeightCacheEntries || g_weights_bytes + e.dev_bytes > kWeightCacheBytes)) {
+    PreparedWeights e = {bytes, hash, type, C, KN, KH, KW, nullptr, dev_bytes, g_weights_clock};
+    while (!g_weights.empty() && (g_weights.size() >= kWeightCacheEntries || g_weights_bytes + e.dev_bytes > cap)) {
         size_t oldest = 0;
         for (size_t i = 1; i < g_weights.size(); i++)
             if (g_weights[i].last_use < g_weights[oldest].last_use) oldest = i;
-        hip_or_die(hipStreamSynchronize(host_stream()), "hipStreamSynchronize");
-        hip_or_die(hipFree(g_weights[oldest].dev), "hipFree");
-        g_weights_bytes -= g_weights[oldest].dev_bytes;
-        g_weights.erase(g_weights.begin() + (long)oldest);
+        drop_weight_entry(oldest);
     }
     hip_or_die(hipMalloc(&e.dev, e.dev_bytes ? e.dev_bytes : 16), "hipMalloc");
     int64_t* d_rows = (int64_t*)upload(SLOT_W, host, bytes);
@@ -618,6 +671,41 @@ static int64_t* host_quantize_im2row(bool ternary, float* x, float* thr, int N, 
     if (ftnn_quantize_im2row(ternary, d_x, d_thr, N, C, H, W, H_pad, W_pad, kH, kW, H_stride,
                              W_stride, d_rows, d_scr, host_stream()) != FTNN_OK)
         die(ternary ? "t2r_p2_opt" : "b2r");
+    int64_t* out = (int64_t*)host_alloc(out_bytes, true);
+    download(out, d_rows, out_bytes);
+    return out;
+}
+
+// the reference's weight packers (src/utils.c:468-521, 634-675) on host pointers: fp32 (KN, C, KH, KW) up, the device
+// packer, Packing-2 rows down into aligned_alloc(32, ...) memory as the reference returns it
+static int64_t* host_pack_weights(bool ternary, float* w, float* thr, int KN, int C, int KH, int KW) {
+    std::lock_guard<std::mutex> lock(g_ctx_mutex);
+    const char* who = ternary ? "ternarize_opt_avx2" : "binarize_opt_avx2";
+    if (KN <= 0 || C <= 0 || KH <= 0 || KW <= 0 || !row_fits(C, KH, KW) || !w || !thr) {
+        fail(FTNN_EINVAL, "non-positive dimension, null pointer or more than %d words per row", kMaxRowWords);
+        die(who);
+    }
+    const size_t out_bytes = (size_t)KN * (size_t)ftnn_row_words(C, KH, KW, ternary) * sizeof(int64_t);
+    float* d_w = (float*)upload(SLOT_X, w, (size_t)KN * C * KH * KW * sizeof(float));
+    float* d_thr = (float*)upload(SLOT_THR, thr, (size_t)KN * sizeof(float));
+    int64_t* d_rows = (int64_t*)dev_buf(SLOT_ROWS, out_bytes);
+    if (ftnn_pack_weights(ternary, d_w, d_thr, KN, C, KH, KW, d_rows, host_stream()) != FTNN_OK) die(who);
+    int64_t* out = (int64_t*)host_alloc(out_bytes, true);
+    download(out, d_rows, out_bytes);
+    return out;
+}
+
+// bitpacking2 (src/utils.c:257-291) on host pointers
+static int64_t* host_pack_gemm_operand(float* x, int I, int J) {
+    std::lock_guard<std::mutex> lock(g_ctx_mutex);
+    if (I <= 0 || J <= 0 || J % 256 != 0 || !x) {   // the reference asserts J % 256 == 0 (src/utils.c:258)
+        fail(FTNN_EINVAL, "bitpacking2: I = %d, J = %d (J must be a positive multiple of 256)", I, J);
+        die("bitpacking2");
+    }
+    const size_t out_bytes = (size_t)I * J / 32 * sizeof(int64_t);
+    float* d_x = (float*)upload(SLOT_X, x, (size_t)I * J * sizeof(float));
+    int64_t* d_rows = (int64_t*)dev_buf(SLOT_ROWS, out_bytes);
+    if (ftnn_pack_gemm_operand(d_x, I, J, d_rows, host_stream()) != FTNN_OK) die("bitpacking2");
     int64_t* out = (int64_t*)host_alloc(out_bytes, true);
     download(out, d_rows, out_bytes);
     return out;
@@ -1294,6 +1382,38 @@ void tnns_conv(testcase_t* t) {
                 T1 - T0, T2 - T1, T3 - T2, T4 - T3, T5 - T4, T5 - T0);
     t->output = y;  // src/tnns/tnns_cpu_mm_p2.c:119
 }
+
+int64_t* ternarize_opt_avx2(float* x, float* q_thresholds, int N, int C, int H, int W) {
+    return host_pack_weights(true, x, q_thresholds, N, C, H, W);
+}
+
+int64_t* binarize_opt_avx2(float* x, float* q_thresholds, int N, int C, int H, int W) {
+    return host_pack_weights(false, x, q_thresholds, N, C, H, W);
+}
+
+int64_t* bitpacking2(float* x, int I, int J) { return host_pack_gemm_operand(x, I, J); }
+
+void ftnn_host_forget_weights(void) {
+    std::lock_guard<std::mutex> lock(g_ctx_mutex);
+    while (!g_weights.empty()) drop_weight_entry(g_weights.size() - 1);
+}
+
+void ftnn_host_release_spares(void) { SparePool::get().release(); }
+
+int ftnn_host_hash_uses_aes(void) { return hash128_uses_aes() ? 1 : 0; }
+
+void ftnn_host_hash128(const void* data, int64_t bytes, int portable, uint64_t out[2]) {
+    const Hash128 h = portable ? hash128_portable(data, (size_t)bytes, 0) : content_hash(data, (size_t)bytes);
+    out[0] = h.lo;
+    out[1] = h.hi;
+}
+
+int64_t ftnn_host_cached_weight_bytes(void) {
+    std::lock_guard<std::mutex> lock(g_ctx_mutex);
+    return (int64_t)g_weights_bytes;
+}
+
+int64_t ftnn_static_scratch_bytes(void) { return kStaticScratchBytes; }
 
 void tnns_gemm(testcase_tnns_gemm_t* t) {
     // alpha is fixed to 1 (src/tnns/tnns_cpu_mm_p2.c:123)

@@ -1201,13 +1201,13 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
     // alone do that (a tile = 64 kernels x 64 pixels)
     const int64_t tiles = ((M + 63) / 64) * ((KN + 63) / 64);
     int split = tiles >= 600 ? 1 : (tiles >= 450 ? 2 : 4);   // measured on MI355X (1024 SIMDs)
-    while (split > 1 && cg.K < split) split /= 2;   // no wavefront without K words of its own
     static const int tune = []() {   // tuning aid: force the K split (1, 2 or 4; anything else is ignored)
         const char* e = getenv("FTNN_CONV_SPLIT");
         const int v = e ? atoi(e) : 0;
         return (v == 1 || v == 2 || v == 4) ? v : 0;
     }();
     if (tune) split = tune;
+    while (split > 1 && cg.K < split) split /= 2;   // no wavefront without K words of its own, forced or not
     const int wpb = 4, tpb = wpb / split;   // wavefronts and pixel tiles per workgroup (see the kernel)
     // few 64 x 64 tiles: tiles of 32 x 32, four times the workgroups (k_conv_f4_small)
     static const int small_below = getenv("FTNN_CONV_SMALL_BELOW") ? atoi(getenv("FTNN_CONV_SMALL_BELOW")) : 150;

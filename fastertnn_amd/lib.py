@@ -61,8 +61,22 @@ _L.mm_bnn.restype = _vp
 _L.mm_bnn.argtypes = [_vp, _vp] + [C.c_int] * 6 + [C.c_float]
 _L.tnns_conv.restype = None
 _L.tnns_gemm.restype = None
+_L.bitpacking2.restype = _vp
+_L.bitpacking2.argtypes = [_vp, C.c_int, C.c_int]
+for _n in ("ternarize_opt_avx2", "binarize_opt_avx2"):
+    getattr(_L, _n).restype = _vp
+    getattr(_L, _n).argtypes = [_vp, _vp] + [C.c_int] * 4
+_L.ftnn_host_forget_weights.restype = None
+_L.ftnn_host_release_spares.restype = None
+_L.ftnn_host_cached_weight_bytes.restype = C.c_int64
+_L.ftnn_host_hash128.restype = None
+_L.ftnn_host_hash128.argtypes = [_vp, C.c_int64, C.c_int, C.POINTER(C.c_uint64)]
+_L.ftnn_static_scratch_bytes.restype = C.c_int64
 
 EXPORTS = ("tnns_conv", "tnns_gemm", "t2r_p2_opt", "b2r", "mm_tnn", "mm_tbn", "mm_btn", "mm_bnn",
+           "bitpacking2", "ternarize_opt_avx2", "binarize_opt_avx2", "ftnn_host_forget_weights",
+           "ftnn_host_release_spares", "ftnn_host_cached_weight_bytes", "ftnn_host_hash128", "ftnn_host_hash_uses_aes",
+           "ftnn_static_scratch_bytes",
            "ftnn_last_error", "ftnn_version", "ftnn_out_dim", "ftnn_row_words",
            "ftnn_pack_scratch_bytes", "ftnn_quantize_im2row", "ftnn_mm", "ftnn_conv",
            "ftnn_pack_weights", "ftnn_pack_gemm_operand", "ftnn_select_engine", "ftnn_mm_scratch_bytes",
@@ -212,7 +226,7 @@ def conv(typ, x, thr, qw, kn, kh, kw, pad, stride, alpha, scratch=None, out=None
     return out
 
 
-STATIC_SCRATCH_BYTES = 32 << 20
+STATIC_SCRATCH_BYTES = int(_L.ftnn_static_scratch_bytes())   # FTNN_STATIC_SCRATCH_BYTES of the build
 
 
 def conv_static(typ, x, thr, qw, kn, kh, kw, pad, stride, alpha, out):
@@ -386,6 +400,37 @@ def host_conv(typ, x, thr, qw, kn, kh, kw, pad, stride, alpha):
     _L.tnns_conv(C.byref(t))
     oh, ow = out_dim(h, pad, kh, stride), out_dim(w, pad, kw, stride)
     return _take(t.output, n * kn * oh * ow, np.float32).reshape(n, kn, oh, ow)
+
+
+def host_pack_weights(w, thr, ternary):
+    """ternarize_opt_avx2 / binarize_opt_avx2 on host pointers: fp32 (KN, C, KH, KW) -> Packing-2 rows"""
+    w, thr = _np(w, np.float32), _np(thr, np.float32)
+    kn, c, kh, kw = w.shape
+    fn = _L.ternarize_opt_avx2 if ternary else _L.binarize_opt_avx2
+    return _take(fn(w.ctypes.data, thr.ctypes.data, kn, c, kh, kw), kn * row_words(c, kh, kw, ternary), np.int64)
+
+
+def host_pack_gemm_operand(x):
+    """bitpacking2 on host pointers: fp32 [I][J] of {-1, 0, +1} -> Packing 2"""
+    x = _np(x, np.float32)
+    i, j = x.shape
+    return _take(_L.bitpacking2(x.ctypes.data, i, j), i * j // 32, np.int64)
+
+
+def host_hash128(a, portable=False):
+    """the prepared-weight cache's content hash of a numpy array's bytes, as (low, high)"""
+    a = np.ascontiguousarray(a)
+    out = (C.c_uint64 * 2)()
+    _L.ftnn_host_hash128(a.ctypes.data, a.nbytes, int(portable), out)
+    return int(out[0]), int(out[1])
+
+
+def host_forget_weights():
+    _L.ftnn_host_forget_weights()
+
+
+def host_cached_weight_bytes():
+    return int(_L.ftnn_host_cached_weight_bytes())
 
 
 def host_gemm(xp, wp, m, n, p_packed, into=None):

@@ -106,6 +106,33 @@ FTNN_API float *mm_btn(int64_t *a, int64_t *b, int N, int OH, int OW, int KN, in
 FTNN_API float *mm_bnn(int64_t *a, int64_t *b, int N, int OH, int OW, int KN, int K, int K_unpack,
               float prelu_alpha);
 
+/* include/utils.h:17,22,26; src/utils.c:257-291, 468-521, 634-675: the packers the reference's drivers prepare their
+ * operands with (src/timing_gemm.c:102-103, src/timing_layers.c:131-134), on host pointers.  bitpacking2 packs an fp32
+ * [I][J] matrix of {-1, 0, +1} into Packing 2 (J a multiple of 256); ternarize_opt_avx2 / binarize_opt_avx2 pack fp32
+ * weights (N, C, H, W) = (kernels, channels, kernel height, kernel width) with one threshold per kernel.  Each
+ * returns aligned_alloc(32, ...) memory that the caller free()s.  A driver that links the reference's own utils.o
+ * keeps the reference's definitions (the executable's symbols come first); to take these instead, compile that one
+ * file with the three names renamed (INTEGRATION.md shows the line). */
+FTNN_API int64_t *bitpacking2(float *x, int I, int J);
+FTNN_API int64_t *ternarize_opt_avx2(float *x, float *q_thresholds, int N, int C, int H, int W);
+FTNN_API int64_t *binarize_opt_avx2(float *x, float *q_thresholds, int N, int C, int H, int W);
+
+/* State behind the host entry points above (no counterpart in the reference, whose functions keep none).
+ * tnns_conv keeps the weights of the layers it has seen on the device in engine form, found again by a 128-bit hash
+ * of their contents, their size and the layer shape (never by address): ftnn_host_forget_weights() frees them all;
+ * FTNN_HOST_NO_WEIGHT_CACHE=1 in the environment keeps none, FTNN_HOST_WEIGHT_CACHE_MB=n caps them (default 1024);
+ * rows beyond 16 MiB are never kept.  Large results are prepared ahead of time by a helper thread once a size
+ * repeats (at most 512 MiB waiting, each dropped after 256 large results have passed it by):
+ * ftnn_host_release_spares() frees those that are ready and forgets the sizes seen. */
+FTNN_API void ftnn_host_forget_weights(void);
+FTNN_API void ftnn_host_release_spares(void);
+/* device bytes the weight cache holds now */
+FTNN_API int64_t ftnn_host_cached_weight_bytes(void);
+/* the cache's content hash of `bytes` bytes (out[0] low, out[1] high half); portable != 0 forces the implementation
+ * without AES instructions on one thread; ftnn_host_hash_uses_aes() says which one the cache uses on this CPU */
+FTNN_API void ftnn_host_hash128(const void *data, int64_t bytes, int portable, uint64_t out[2]);
+FTNN_API int ftnn_host_hash_uses_aes(void);
+
 /* ------------------------------------------- 2. device-memory entry points */
 
 #define FTNN_OK 0
@@ -218,14 +245,16 @@ FTNN_API int ftnn_conv(int type, const float *d_x, const float *d_thr, const int
  * ftnn_conv without a scratch argument and without any allocation.  No counterpart in the reference; it is for
  * callers that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc.  The layer's work space (the quantised input and the weights in engine form) is a fixed array
- * of FTNN_STATIC_SCRATCH_BYTES inside the library's code object, which every GPU the library runs on holds from
- * the first call until the process ends.  A layer whose ftnn_conv_scratch_bytes() exceeds that is refused with
+ * of FTNN_STATIC_SCRATCH_BYTES inside the library's code object: every GPU on which the process loads the library's
+ * code holds its copy from that load until the process ends, whether or not the entry point is ever called
+ * (ftnn_static_scratch_bytes() returns the size the library was built with).  A layer whose ftnn_conv_scratch_bytes() exceeds that is refused with
  * FTNN_EINVAL.  The call itself performs no hipMalloc / hipFree and synchronises nothing; the first call on a
  * device looks the array's address up (hipGetSymbolAddress), so make that first call outside a graph capture.
  * All calls on one GPU share the one array: calls that overlap on a GPU (two streams, two threads) race, and the
  * array keeps the last call's contents (every call overwrites the part it reads).  Same result as ftnn_conv.
  */
 #define FTNN_STATIC_SCRATCH_BYTES (32 << 20)
+FTNN_API int64_t ftnn_static_scratch_bytes(void);
 FTNN_API int ftnn_conv_static(int type, const float *d_x, const float *d_thr, const int64_t *d_qw, int N, int C,
                               int H, int W, int KN, int KH, int KW, int H_pad, int W_pad, int H_stride,
                               int W_stride, float prelu_alpha, float *d_y, void *stream);

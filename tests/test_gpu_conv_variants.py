@@ -24,10 +24,11 @@ from tests.cases import make_layer
 from tests.test_gpu_net import STACK, STACK2, STACK3, build, oracle_chain
 oracle = Oracle()
 # single layers with an fp32 result: 256 tiles of 64 x 64 (the 64 x 64 kernel, split as forced), 8 tiles (32 x 32
-# tiles), ragged kernel counts and pixel counts, a strided window
+# tiles), ragged kernel counts and pixel counts, a strided window, and 1 x 1 layers of one and two K words on more
+# than 150 tiles of 64 x 64 (a forced split of 2 or 4 must not leave a wavefront without a word of its own)
 for typ in range(4):
     for shape, batch in (((64, 32, 32, 128, 3, 3, 1, 1), 8), ((130, 17, 17, 70, 3, 3, 1, 2), 21), ((64, 10, 10, 64, 3, 3, 1, 1), 2),
-                         ((200, 6, 7, 33, 1, 1, 0, 1), 3)):
+                         ((200, 6, 7, 33, 1, 1, 0, 1), 3), ((64, 40, 40, 64, 1, 1, 0, 1), 11), ((100, 24, 24, 96, 1, 1, 0, 2), 40)):
         L = make_layer(typ, shape, batch, seed=8000 + typ)
         print("case", TYPE_NAMES[typ], shape, batch, flush=True)
         wt = weight_is_ternary(typ)

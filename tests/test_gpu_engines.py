@@ -201,6 +201,7 @@ def test_vector_alu_gemm_splits_k_for_small_problems(hip, oracle, typ, shape):
 
 _KSPLIT_CHILD = r"""
 import sys
+import torch    # before the library, as in every other test process: both then share torch's HIP runtime
 sys.path.insert(0, sys.argv[1])
 import fastertnn_amd.lib as hip
 from oracle.ftnn_oracle import Oracle

@@ -114,3 +114,33 @@ def test_reference_gemm_driver(tmp_path):
     run([REF_GEMM, "final"], tmp_path, timeout=560)
     header, rows = read_csv(tmp_path / "out" / "measurements" / "gemm")
     assert header == ["m", "n", "p", "Runtime", "Type"] and [int(r[0]) for r in rows] == [32, 64, 128, 256, 512, 1024, 2048, 4096]
+
+
+# ---- the same drivers with the reference's operand packers (bitpacking2, ternarize_opt_avx2, binarize_opt_avx2) taken
+# from the library as well: the reference's utils.c compiled with those three names renamed (oracle/Makefile) ----
+REF_LAYERS_DEVPACK = REF_LAYERS + "_devpack"
+REF_GEMM_DEVPACK = REF_GEMM + "_devpack"
+
+
+@pytest.mark.parametrize("net", ["tnn", "tbn", "btn", "bnn"])
+def test_reference_self_test_with_the_librarys_weight_packers(net, tmp_path):
+    """the driver packs its weights with the library's ternarize_opt_avx2 / binarize_opt_avx2, runs tnns_conv on them and
+    abort()s unless the result equals its fp32 direct convolution (src/timing_layers.c:127-165)"""
+    _need(REF_LAYERS_DEVPACK)
+    os.makedirs(tmp_path / "out" / "measurements")
+    out = run([REF_LAYERS_DEVPACK, "final", net, "test"], tmp_path)
+    assert "SHAPE 11" in out
+
+
+def test_reference_gemm_driver_with_the_librarys_bitpacking2(tmp_path):
+    """the sweep up to 4096 x 4096 x 32768 with both operands of every size packed by the library's bitpacking2 (the
+    reference's scalar packer takes seconds on the largest); wall time of both forms is printed"""
+    import time
+    _need(REF_GEMM_DEVPACK)
+    os.makedirs(tmp_path / "out" / "measurements" / "gemm")
+    t0 = time.perf_counter()
+    run([REF_GEMM_DEVPACK, "final"], tmp_path, timeout=560)
+    dt = time.perf_counter() - t0
+    header, rows = read_csv(tmp_path / "out" / "measurements" / "gemm")
+    assert header == ["m", "n", "p", "Runtime", "Type"] and [int(r[0]) for r in rows] == [32, 64, 128, 256, 512, 1024, 2048, 4096]
+    print("reference GEMM driver with the library's bitpacking2: %.2f s of wall time" % dt)

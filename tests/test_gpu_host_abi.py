@@ -242,3 +242,116 @@ def test_copy_sizes_around_the_staging_chunks(hip, oracle, pixels):
     for rep in range(2):
         got = hip.host_conv(TBN, L["x"], L["thr"], qw, kn, 1, 1, 0, 1, 0.5)
         assert got.tobytes() == want.tobytes(), rep
+
+
+def test_same_rows_at_another_address_are_found_again(hip, oracle):
+    """the prepared-weight cache knows a layer by the contents of its rows, their size and the layer shape, not by where
+    they lie: a caller that packs the same weights again into fresh memory (the reference's e2e driver packs per layer
+    and pass) adds no entry; different rows do; ftnn_host_forget_weights() drops them all"""
+    L = make_layer(TNN, (128, 9, 9, 96, 3, 3, 1, 1), 2, seed=7100)
+    q = oracle.pack_weights(L["w"], L["wthr"], True)
+    want = oracle.conv(TNN, L["x"], L["thr"], q, L["kn"], 3, 3, 1, 1, 0.5).reshape(-1)
+    hip.host_forget_weights()
+    assert hip.host_cached_weight_bytes() == 0
+    assert _conv_at(hip, TNN, L, q).tobytes() == want.tobytes()
+    held = hip.host_cached_weight_bytes()
+    assert held > 0
+    for rep in range(3):
+        other = np.empty(q.size + 8 * rep + 8, np.int64)[8 * rep + 4:][:q.size]      # another address every time
+        other[:] = q
+        assert other.ctypes.data != q.ctypes.data
+        assert _conv_at(hip, TNN, L, other).tobytes() == want.tobytes()
+        assert hip.host_cached_weight_bytes() == held, "identical rows must not add an entry"
+    q2 = q.copy()
+    q2[5] ^= 1 << 40
+    want2 = oracle.conv(TNN, L["x"], L["thr"], q2, L["kn"], 3, 3, 1, 1, 0.5).reshape(-1)
+    assert _conv_at(hip, TNN, L, q2).tobytes() == want2.tobytes()
+    assert hip.host_cached_weight_bytes() == 2 * held
+    hip.host_forget_weights()
+    assert hip.host_cached_weight_bytes() == 0
+    assert _conv_at(hip, TNN, L, q).tobytes() == want.tobytes()       # and the layer still runs
+    assert hip.host_cached_weight_bytes() == held
+
+
+def test_weight_rows_beyond_16_mib_are_not_kept(hip, oracle):
+    """rows of more than 16 MiB are uploaded and prepared on every call (reading them once on the host to hash them
+    costs what the upload costs); the result is the same and the cache does not grow"""
+    c, kn, n = 16384, 4100, 2
+    rng = np.random.default_rng(72)
+    q = rng.integers(-2 ** 63, 2 ** 63, size=kn * 2 * (c // 64), dtype=np.int64)
+    assert q.nbytes > 16 << 20
+    x = rng.standard_normal((n, c, 1, 1)).astype(np.float32)
+    thr = np.full(n, 0.5, np.float32)
+    L = dict(x=x, thr=thr, c=c, ih=1, iw=1, kn=kn, kh=1, kw=1, pad=0, stride=1)
+    want = oracle.conv(TNN, x, thr, q, kn, 1, 1, 0, 1, 0.5).reshape(-1)
+    hip.host_forget_weights()
+    for rep in range(2):
+        assert _conv_at(hip, TNN, L, q).tobytes() == want.tobytes(), rep
+        assert hip.host_cached_weight_bytes() == 0
+    q[11] ^= 1 << 3                                    # rewritten in place: nothing stale can be served
+    want = oracle.conv(TNN, x, thr, q, kn, 1, 1, 0, 1, 0.5).reshape(-1)
+    assert _conv_at(hip, TNN, L, q).tobytes() == want.tobytes()
+
+
+_NO_CACHE_CHILD = r"""
+import sys
+import numpy as np, torch
+sys.path.insert(0, sys.argv[1])
+import fastertnn_amd.lib as hip
+from fastertnn_amd import TNN
+from oracle.ftnn_oracle import Oracle
+from tests.cases import make_layer
+oracle = Oracle()
+L = make_layer(TNN, (128, 9, 9, 96, 3, 3, 1, 1), 2, seed=7100)
+q = oracle.pack_weights(L["w"], L["wthr"], True)
+want = oracle.conv(TNN, L["x"], L["thr"], q, L["kn"], 3, 3, 1, 1, 0.5)
+for rep in range(3):
+    got = hip.host_conv(TNN, L["x"], L["thr"], q, L["kn"], 3, 3, 1, 1, 0.5)
+    assert got.tobytes() == want.tobytes(), rep
+    assert hip.host_cached_weight_bytes() == int(sys.argv[2]) * (rep >= 0), hip.host_cached_weight_bytes()
+print("child ok")
+"""
+
+
+@pytest.mark.parametrize("env", [{"FTNN_HOST_NO_WEIGHT_CACHE": "1"}, {"FTNN_HOST_WEIGHT_CACHE_MB": "0"}])
+def test_weight_cache_switched_off(env):
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    print("case weight cache off", env, flush=True)
+    r = subprocess.run([sys.executable, "-c", _NO_CACHE_CHILD, root, "0"], env=dict(os.environ, **env), capture_output=True,
+                       text=True, timeout=110)
+    assert r.returncode == 0 and "child ok" in r.stdout, r.stdout[-1500:] + r.stderr[-1500:]
+
+
+@pytest.mark.parametrize("ternary", [True, False], ids=["ternarize_opt_avx2", "binarize_opt_avx2"])
+def test_host_weight_packers(hip, oracle, ternary):
+    """the reference's weight packers on host pointers (src/utils.c:468-521, 634-675) against the oracle's restatement,
+    word for word: channel tails, padding words, thresholds of either sign, a tensor beyond the 4 MiB staging chunks"""
+    from fastertnn_amd import synth
+    for shape in ((5, 3, 7, 7), (64, 64, 3, 3), (33, 65, 1, 1), (130, 127, 3, 3), (300, 1024, 2, 2)):
+        kn, c, kh, kw = shape
+        print("case host weight packer", ternary, shape, flush=True)
+        w = synth.normal(kn * 31 + c, shape)
+        for thr_value in (0.5, 0.0, -0.25):
+            thr = np.full(kn, thr_value, np.float32)
+            thr[::2] *= 0.5
+            want = oracle.pack_weights(w, thr, ternary)
+            got = hip.host_pack_weights(w, thr, ternary)
+            assert got.tobytes() == np.ascontiguousarray(want).tobytes(), (shape, thr_value)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 256), (3, 1280), (257, 4096), (600, 8192)])
+def test_host_bitpacking2(hip, oracle, rows, cols):
+    """bitpacking2 on host pointers (src/utils.c:257-291) against the oracle's, word for word; the last case moves 19 MB
+    through the staging ring"""
+    from fastertnn_amd import synth
+    x = synth.ternary(rows * 7 + cols, (rows, cols))
+    want = oracle.pack_gemm_operand(x)
+    got = hip.host_pack_gemm_operand(x)
+    assert got.tobytes() == np.ascontiguousarray(want).tobytes()
+    # values outside {-1, 0} count as +1 (neither bit), as in the reference's if / else if
+    x2 = x.copy()
+    x2[0, :7] = (2.0, -3.0, 0.5, -0.0, 1e-30, -1.0, 7.0)
+    assert hip.host_pack_gemm_operand(x2).tobytes() == np.ascontiguousarray(oracle.pack_gemm_operand(x2)).tobytes()
