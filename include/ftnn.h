@@ -120,8 +120,8 @@ FTNN_API int64_t *binarize_opt_avx2(float *x, float *q_thresholds, int N, int C,
 /* State behind the host entry points above (no counterpart in the reference, whose functions keep none).
  * tnns_conv keeps the weights of the layers it has seen on the device in engine form, found again by a 128-bit hash
  * of their contents, their size and the layer shape (never by address): ftnn_host_forget_weights() frees them all;
- * FTNN_HOST_NO_WEIGHT_CACHE=1 in the environment keeps none, FTNN_HOST_WEIGHT_CACHE_MB=n caps them (default 1024);
- * rows beyond 16 MiB are never kept.  Large results are prepared ahead of time by a helper thread once a size
+ * FTNN_HOST_NO_WEIGHT_CACHE=1 in the environment keeps none, FTNN_HOST_WEIGHT_CACHE_MB=n caps them (default 1024;
+ * a layer whose prepared weights alone exceed the cap is uploaded and prepared on every call).  Large results are prepared ahead of time by a helper thread once a size
  * repeats (at most 512 MiB waiting, each dropped after 256 large results have passed it by):
  * ftnn_host_release_spares() frees those that are ready and forgets the sizes seen. */
 FTNN_API void ftnn_host_forget_weights(void);

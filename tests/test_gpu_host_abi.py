@@ -273,9 +273,9 @@ def test_same_rows_at_another_address_are_found_again(hip, oracle):
     assert hip.host_cached_weight_bytes() == held
 
 
-def test_weight_rows_beyond_16_mib_are_not_kept(hip, oracle):
-    """rows of more than 16 MiB are uploaded and prepared on every call (reading them once on the host to hash them
-    costs what the upload costs); the result is the same and the cache does not grow"""
+def test_large_weight_rows_are_hashed_in_slices_and_kept(hip, oracle):
+    """rows of 17 MiB: hashed in slices on the copy threads, kept like any other layer's, and a single flipped bit
+    anywhere in them is seen"""
     c, kn, n = 16384, 4100, 2
     rng = np.random.default_rng(72)
     q = rng.integers(-2 ** 63, 2 ** 63, size=kn * 2 * (c // 64), dtype=np.int64)
@@ -287,10 +287,14 @@ def test_weight_rows_beyond_16_mib_are_not_kept(hip, oracle):
     hip.host_forget_weights()
     for rep in range(2):
         assert _conv_at(hip, TNN, L, q).tobytes() == want.tobytes(), rep
-        assert hip.host_cached_weight_bytes() == 0
-    q[11] ^= 1 << 3                                    # rewritten in place: nothing stale can be served
-    want = oracle.conv(TNN, x, thr, q, kn, 1, 1, 0, 1, 0.5).reshape(-1)
-    assert _conv_at(hip, TNN, L, q).tobytes() == want.tobytes()
+    held = hip.host_cached_weight_bytes()
+    assert held > 0
+    for pos in (11, q.size // 2 + 3, q.size - 2):      # rewritten in place, in the first, a middle and the last slice
+        q[pos] ^= 1 << 3
+        want = oracle.conv(TNN, x, thr, q, kn, 1, 1, 0, 1, 0.5).reshape(-1)
+        assert _conv_at(hip, TNN, L, q).tobytes() == want.tobytes(), pos
+    assert hip.host_cached_weight_bytes() == 4 * held
+    hip.host_forget_weights()
 
 
 _NO_CACHE_CHILD = r"""
@@ -315,6 +319,7 @@ print("child ok")
 
 @pytest.mark.parametrize("env", [{"FTNN_HOST_NO_WEIGHT_CACHE": "1"}, {"FTNN_HOST_WEIGHT_CACHE_MB": "0"}])
 def test_weight_cache_switched_off(env):
+    """with the cache off (or capped below the layer's prepared weights) every call uploads and prepares its weights"""
     import os
     import subprocess
     import sys
