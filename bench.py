@@ -3,12 +3,12 @@
 
 Headline workload: the large compute-bound TNN GEMM (M = N = 8192, K = 32768,
 uniform ternary operands in Packing 2, PReLU(0.5) fused).  One "step" is one pass of
-the GEMM over one batch of activation rows, everything resident in HBM: the packed
-activation operand A is turned into matrix-core fragments (ftnn_expand_rows) and
-multiplied with the weights B, which were brought into that form once before the timed
-region, as a layer keeps them (ftnn_mm_expanded).  Where the library's engine choice
-for the shape is the vector ALU the step is the one call ftnn_mm_engine.  Prints ONE
-JSON line:
+the GEMM from two PACKED operands resident in HBM, as the reference's mm_tnn takes
+them: both are brought into the engine's operand form (ftnn_expand_rows) and
+multiplied (ftnn_mm_expanded) -- the launches of one ftnn_mm_engine call.  Where the
+library's engine choice for the shape is the vector ALU the step is that one call.
+The step of a layer that keeps its weights in engine form is reported beside it
+(step_with_weights_kept_in_engine_form).  Prints ONE JSON line:
 
   value        ternary GMAC/s = M*N*K / time of a step
   roofline     the dominant kernel of the step (the fp4 matrix-core GEMM): its launches
@@ -25,7 +25,10 @@ JSON line:
                operands, or the AVX2 restatement under oracle/ where that build is
                absent; the GPU rows of the sample are compared bit-for-bit
   extra        conv-layer and layer-chain latencies (kernel-only and host-pointer ABI
-               inclusive); --full adds the reference's sweeps and tables
+               inclusive), the other types on the headline shape, the reference's GEMM
+               sweep, its 17 single layers and two of its networks, each with a roofline
+               object and a bit-for-bit comparison with the reference's CPU path; --full
+               adds the other networks, batch sizes and types
 """
 import argparse
 import json
@@ -38,6 +41,28 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 VALU_PEAK_TOPS = 256 * 4 * 16 * 2.4e9 / 1e12  # 39.32 T lane-ops/s (int32 VALU, one op per lane per clock)
+
+
+MFMA_F4_PEAK_TFLOPS = 10100.0   # dense fp4 matrix rate of MI355X
+
+
+def roofline_mfma_f4(macs, ms):
+    """roofline object of a kernel (or chain of kernels) on the fp4 matrix cores: 2 FLOP per lane-MAC"""
+    ach = 2.0 * macs / (ms * 1e-3) / 1e12
+    return {"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_F4_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(ach / MFMA_F4_PEAK_TFLOPS, 4)}
+
+
+def roofline_valu(m, n, kw, ms, ops_per_pair=4):
+    """roofline object of the vector-ALU popcount GEMM: ops_per_pair lane-ops per pair of 32-lane dwords (4 for TNN, 2
+    for the types with a binary operand) against 256 CU x 4 SIMD x 16 lanes x 2.4 GHz"""
+    ach = float(ops_per_pair) * m * n * (2 * kw) / (ms * 1e-3) / 1e12
+    return {"bound": "valu", "achieved": round(ach, 3), "peak": round(VALU_PEAK_TOPS, 3), "unit": "Tlaneop/s",
+            "frac": round(ach / VALU_PEAK_TOPS, 4)}
+
+
+def roofline_for(engine_name, m, n, kw, ms, ops_per_pair=4):
+    return roofline_mfma_f4(float(m) * n * kw * 64, ms) if engine_name == "mfma_f4" else roofline_valu(m, n, kw, ms, ops_per_pair)
 
 
 def parse():
@@ -189,6 +214,8 @@ def small_gemm(torch, lib, m, n, k, reps=30):
         tg, same = graph_times(torch, run, y, reps)
         out[name] = {"call_ms": round(t, 4), "gmacs": round(float(m) * n * k / t / 1e6, 1), "bit_exact_vs_cpu": exact,
                      "device_ms_in_a_graph_of_10_calls": round(tg, 4), "graph_replays_same_bits_as_eager": same}
+        if name != "mfma_i8":   # whole call (expansions included for fp4) over the device time of a call in the graph
+            out[name]["roofline"] = roofline_for(name, m, n, kw, tg)
     t_abi = []
     for _ in range(10):
         t0 = time.perf_counter()
@@ -229,6 +256,9 @@ def other_types(torch, lib, a_tern, b_tern, m, n, k, reps=5):
             t = sum(t) / len(t)
             row[en] = {"call_ms": round(t, 4), "gmacs": round(float(m) * n * k / t / 1e6, 1), "same_bits_as_valu": same}
         row["valu_roofline_frac"] = round(2.0 * m * n * 2 * kw / (row["valu"]["call_ms"] * 1e-3) / 1e12 / VALU_PEAK_TOPS, 4)
+        row["valu"]["roofline"] = roofline_valu(m, n, kw, row["valu"]["call_ms"], 2)
+        row["mfma_f4"]["roofline"] = roofline_mfma_f4(float(m) * n * k, row["mfma_f4"]["call_ms"])
+        row["all_engines_same_bits"] = all(r["same_bits_as_valu"] for r in (row["valu"], row["mfma_i8"], row["mfma_f4"]))
         out[name] = row
         del scratch, first
     return out
@@ -321,6 +351,8 @@ def conv_latency(torch, lib, typ, shape, batch, seed, reps=20):
            "engine": lib.ENGINE_NAMES[lib.select_conv_engine(typ, batch, c, ih, iw, kn, kh, kw, pad, stride)],
            "abi_ms": round(sorted(t)[7], 3),
            "gmacs_kernel": round(batch * oh * ow * kn * c * kh * kw / kernel_ms / 1e6, 1)}
+    out["roofline"] = roofline_for(out["engine"], batch * oh * ow, kn, ((c + 63) // 64) * kh * kw, kernel_ms,
+                                   4 if typ == 0 else 2)
     # the reference's layer on one host core, same inputs
     from oracle import ftnn_oracle as O
     if O.Reference.available():
@@ -386,6 +418,8 @@ def e2e_latency(torch, lib, batch, reps=50, cpu=True, typ=None):
             t10 = sorted(event_times(torch, ten, max(5, reps // 2)))[max(5, reps // 2) // 2] / 10
             out[key.replace("_ms", "_ms_per_pass_of_ten_queued")] = round(t10, 4)
     st.synchronize()
+    # the chain's layers run on the fp4 matrix cores: logical MACs of the whole pass over its device time
+    out["roofline"] = roofline_mfma_f4(macs, out["eager_ms_per_pass_of_ten_queued"])
     from oracle import ftnn_oracle as O
     if cpu and O.Reference.available():
         ref = O.Reference()
@@ -451,6 +485,33 @@ class Probe:
         """shader clock seen by a short, nearly idle kernel queued directly behind whatever ran last on the stream"""
         r = self._call(self.lib.probe_clock_run, trips, torch, 2)
         return None if r is None else {"ms": round(r[0], 4), "shader_mhz": round(r[1], 1)}
+
+
+def grid_sync_cost(torch):
+    """bench_probe/libprobe_gridsync.so: microseconds per grid-wide synchronisation inside one cooperative launch (the
+    library's cooperative_groups grid sync, and a counter barrier with a bounded wait) against microseconds per launch
+    boundary of plain launches, 18 synchronisations each (a 19-layer chain), one workgroup of 256 threads per compute
+    unit.  What decides whether a chain of small layers should be one resident kernel."""
+    import ctypes as C
+    path = os.path.join(ROOT, "bench_probe", "libprobe_gridsync.so")
+    if not os.path.exists(path):
+        return {"skipped": "bench_probe/libprobe_gridsync.so is not built"}
+    lib = C.CDLL(path)
+    lib.probe_gridsync_run.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double)]
+    out = {}
+    buf = (C.c_double * 4)()
+    st = torch.cuda.current_stream().cuda_stream
+    for mode, key in ((2, "launch_boundary"), (0, "cooperative_groups_grid_sync"), (1, "counter_barrier_bounded_wait")):
+        best = None
+        for _ in range(5):
+            if lib.probe_gridsync_run(mode, 1, 18, st, buf) != 0:
+                return {"failed": key}
+            if buf[3] != 1.0:
+                return {"failed": key + ": data passed through the synchronisations is wrong"}
+            best = buf[1] if best is None else min(best, buf[1])
+        out[key + "_us"] = round(best, 2)
+        out["workgroups"] = int(buf[2])
+    return out
 
 
 def valu_reconciliation(torch, probe, run_valu, valu_ops, reps=12):
@@ -520,6 +581,9 @@ def reference_gemm_sweep(torch, lib, reps=10):
         t = sorted(event_times(torch, run, reps))[reps // 2]
         row = {"engine": lib.ENGINE_NAMES[lib.select_engine(TNN, m, 1, 1, m, kw)], "device_ms": round(t, 4),
                "gmacs": round(float(m) * m * p / t / 1e6, 1)}
+        tg, same = graph_times(torch, run, y, reps)
+        row["device_ms_in_a_graph_of_10_calls"], row["graph_replays_same_bits_as_eager"] = round(tg, 4), same
+        row["roofline"] = roofline_for(row["engine"], m, m, kw, min(t, tg))
         if O.Reference.available():
             ref = O.Reference()
             ah, bh = O.aligned_copy(a.cpu().numpy()), O.aligned_copy(b.cpu().numpy())
@@ -564,6 +628,9 @@ def reference_single_layers(torch, lib, batch=8, reps=10):
         t = sorted(event_times(torch, step, reps))[reps // 2]
         row = {"engine": lib.ENGINE_NAMES[lib.select_conv_engine(TNN, batch, c, ih, iw, kn, kh, kw, p, s)],
                "device_ms": round(t, 4), "gmac": round(batch * oh * ow * kn * c * kh * kw / 1e9, 2)}
+        tg, same = graph_times(torch, step, y, reps)
+        row["device_ms_in_a_graph_of_10_calls"], row["graph_replays_same_bits_as_eager"] = round(tg, 4), same
+        row["roofline"] = roofline_for(row["engine"], batch * oh * ow, kn, ((c + 63) // 64) * kh * kw, min(t, tg))
         if O.Reference.available():
             ref = O.Reference()
             xh, qwh = x.cpu().numpy(), O.aligned_copy(qw.cpu().numpy())
@@ -576,7 +643,7 @@ def reference_single_layers(torch, lib, batch=8, reps=10):
     return out
 
 
-def reference_networks(torch, lib, batch=8, reps=5):
+def reference_networks(torch, lib, batch=8, reps=5, only=None):
     """the seven networks of the reference's e2e mode (include/timing/shapes_e2e.h, kept as data in
     fastertnn_amd/data/reference_shape_tables.txt), at the reference's batch of 8 (src/timing_layers.c:46): device-resident
     layer chain against the same tnns_conv chain on one host core.  Three tables leave out their pooling layers; there
@@ -591,6 +658,8 @@ def reference_networks(torch, lib, batch=8, reps=5):
     g = torch.Generator(device="cuda")
     g.manual_seed(8)
     for net_t in tables["e2e"]:
+        if only is not None and net_t["name"] not in only:
+            continue
         shapes = [tuple(r) for r in net_t["layers"]]
         c, h, w = shapes[0][:3]
         ok = True
@@ -610,7 +679,8 @@ def reference_networks(torch, lib, batch=8, reps=5):
         t = sorted(event_times(torch, lambda: net.run(x, out=y), reps))[reps // 2]
         macs = sum(batch * lib.out_dim(ih, p, kh, s) * lib.out_dim(iw, p, kw, s) * kn * c * kh * kw
                    for (c, ih, iw, kn, kw, kh, p, s) in shapes)
-        row = {"layers": len(shapes), "gmac": round(macs / 1e9, 1), "device_ms": round(t, 4), "chains_shape_to_shape": ok}
+        row = {"layers": len(shapes), "gmac": round(macs / 1e9, 1), "device_ms": round(t, 4), "chains_shape_to_shape": ok,
+               "roofline": roofline_mfma_f4(macs, t)}
         if O.Reference.available():
             ref = O.Reference()
             xh = x.cpu().numpy()
@@ -686,9 +756,11 @@ def main():
                           dtype=torch.uint8, device="cuda")
     macs = float(m) * n * k
 
-    # The timed hot path.  Matrix-core engines: the weights B are in engine form already (done once, below, outside
-    # the timed region: a layer keeps its weights that way); a step expands the activation rows A and multiplies.
-    # The GEMM kernel of every timed step sits between two HIP events on the launch stream.
+    # The timed hot path: what the reference's mm_tnn does per call -- both operands arrive as packed rows.  On a
+    # matrix-core engine a step therefore brings BOTH operands into engine form (ftnn_expand_rows on A and on B) and
+    # multiplies (ftnn_mm_expanded); these are the launches of the one C call ftnn_mm_engine, issued as three calls so
+    # that the GEMM kernel of every timed step sits between two HIP events on the launch stream.  The cheaper step of a
+    # layer that keeps its weights in engine form (B expanded once) is timed beside it, outside the timed region.
     gemm_events = []
     if auto == lib.ENGINE_VALU:
         def step(timed=False):
@@ -700,12 +772,14 @@ def main():
             if timed:
                 e1.record()
         step_desc = "ftnn_mm_engine (vector ALU) on the packed operands"
+        step_kept = None
     else:
-        b_exp = lib.expand_rows(auto, b, n, kw, True)
+        b_exp = torch.empty(int(lib._L.ftnn_expand_bytes(auto, n, kw)), dtype=torch.uint8, device="cuda")
         a_exp = torch.empty(int(lib._L.ftnn_expand_bytes(auto, m, kw)), dtype=torch.uint8, device="cuda")
 
         def step(timed=False):
             lib.expand_rows(auto, a, m, kw, True, out=a_exp)
+            lib.expand_rows(auto, b, n, kw, True, out=b_exp)
             if timed:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 gemm_events.append((e0, e1))
@@ -713,8 +787,12 @@ def main():
             lib.mm_expanded(auto, TNN, a_exp, b_exp, m, 1, 1, n, kw, alpha, out=y)
             if timed:
                 e1.record()
-        step_desc = ("ftnn_expand_rows(A) + ftnn_mm_expanded with B expanded once before the timed region "
-                     "(weights kept in engine form)")
+
+        def step_kept():
+            lib.expand_rows(auto, a, m, kw, True, out=a_exp)
+            lib.mm_expanded(auto, TNN, a_exp, b_exp, m, 1, 1, n, kw, alpha, out=y)
+        step_desc = ("ftnn_expand_rows(A) + ftnn_expand_rows(B) + ftnn_mm_expanded: both operands from packed rows in "
+                     "every step, as mm_tnn takes them (the launches of one ftnn_mm_engine call)")
 
     if args.copy_calibration:
         src = torch.empty(1 << 26, dtype=torch.float32, device="cuda").fill_(1.0)
@@ -758,6 +836,19 @@ def main():
     gemm_avg = sum(gemm_ms) / len(gemm_ms)
     step_same = bool(torch.equal(y, y_ref))
     del y_ref
+    kept = None
+    if step_kept is not None:
+        # a layer's step: the weights stay in engine form, only the activation rows are expanded per step
+        for _ in range(args.warmup):
+            step_kept()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step_kept()
+        torch.cuda.synchronize()
+        ms_kept = (time.perf_counter() - t0) / args.steps * 1e3
+        kept = {"ms_per_step": round(ms_kept, 4), "gmacs": round(macs / (ms_kept * 1e-3) / 1e9, 1),
+                "step": "ftnn_expand_rows(A) + ftnn_mm_expanded with B expanded once (weights kept in engine form)"}
 
     # the vector-ALU kernel against the roofline the metric names, with the issue-rate probe beside it
     valu_ops = 4.0 * m * n * (2 * kw)      # 4 vector ops per pair of 32-lane dwords, 2*kw dwords per plane
@@ -862,13 +953,14 @@ def main():
             "tnn_resnet18_like_b32_e2e": e2e_latency(torch, lib, 32),
             "quantize_im2row_pack": pack_rates(torch, lib),
             "host_mm_8192x8192x32768": host_gemm_cfg4(torch, lib, a, b, m, n, kw) if (m, n, k) == (8192, 8192, 32768) else None,
+            "other_types_same_gemm_shape": other_types(torch, lib, a, b, m, n, k),
+            "reference_gemm_sweep": reference_gemm_sweep(torch, lib),
+            "reference_single_layers_b8": reference_single_layers(torch, lib),
+            "reference_e2e_networks_b8": reference_networks(torch, lib, only=None if args.full else ("resnet18", "resnet152")),
+            "grid_sync_against_launch_boundary": grid_sync_cost(torch),
         }
         if args.full:
             extra.update({
-                "other_types_same_gemm_shape": other_types(torch, lib, a, b, m, n, k),
-                "reference_gemm_sweep": reference_gemm_sweep(torch, lib),
-                "reference_single_layers_b8": reference_single_layers(torch, lib),
-                "reference_e2e_networks_b8": reference_networks(torch, lib),
                 "tnn_resnet18_like_other_batches": {"b%d" % bb: e2e_latency(torch, lib, bb, cpu=False) for bb in (1, 8, 128)},
                 "other_types_resnet18_like_b32": {nm: e2e_latency(torch, lib, 32, cpu=False, typ=t)
                                                   for nm, t in (("tbn", 1), ("btn", 2), ("bnn", 3))},
@@ -883,6 +975,7 @@ def main():
                    "m": m, "n": n, "k": k, "step": step_desc},
         "roofline": roofline, "cpu_baseline": cpu,
         "engine": lib.ENGINE_NAMES[auto], "step_same_bits_as_valu": step_same,
+        "step_with_weights_kept_in_engine_form": kept,
         "engines_whole_call_from_packed_operands": engines,
         "roofline_mfma_i8_kernel": mfma[lib.ENGINE_MFMA_I8] if auto != lib.ENGINE_MFMA_I8 else None,
         "extra": extra,
