@@ -767,10 +767,13 @@ static int64_t gemm_route_plane_bytes(int N, int C, int H, int W) {
 static int64_t gemm_route_row_bytes(int64_t M, int Kw) { return (M * Kw * 16 + 255) / 256 * 256; }
 
 // operand region of the fp4 layer for this shape, whichever form it takes
-int64_t conv_f4_operand_bytes(int N, int C, int H, int W, int KH, int KW, int OH, int OW, int KN) {
+int64_t conv_f4_operand_bytes(int N, int C, int H, int W, int KH, int KW, int OH, int OW, int KN, int W_stride) {
     if (dense_f4_applies(C, KH, KW)) return conv_f4_dense_bytes(N, C, H, W, KH, KW, OH, OW);
     int64_t bytes = conv_f4_p4_bytes(N, C, H, W);
     const int64_t M = (int64_t)N * OH * OW;
+    // the tile kernel's layout of the same input: a little larger where the width is no multiple of the stride
+    const int64_t t4 = quantize_f4_tiled_bytes(N, C, H, W, W_stride);
+    if (conv_f4_tile_route(M, KN, cpack_of(C), KH * KW, t4, 0, W_stride)) bytes = std::max(bytes, (t4 + 255) / 256 * 256);
     if (conv_f4_gemm_route(M, KN, cpack_of(C) * KH * KW)) {
         const int Kw = conv_f4_weight_words(C, KH, KW);
         const int64_t route = gemm_route_plane_bytes(N, C, H, W) + gemm_route_row_bytes(M, Kw) +
@@ -819,7 +822,8 @@ int conv_f4_expanded(int type, const float* d_x, const float* d_thr, const void*
         return e == hipSuccess ? FTNN_OK : hip_fail(e, "fp4 conv launch");
     }
     const int64_t M = (int64_t)N * OH * OW;
-    if (d_x && qo.mode == 0 && conv_f4_gemm_route(M, KN, cpack_of(C) * KH * KW)) {
+    const bool tiles = d_x && qo.mode == 0 && conv_f4_tile_route(M, KN, cpack_of(C), KH * KW, quantize_f4_tiled_bytes(N, C, H, W, W_stride), W_pad, W_stride);
+    if (d_x && qo.mode == 0 && !tiles && conv_f4_gemm_route(M, KN, cpack_of(C) * KH * KW)) {
         const int Kw = conv_f4_weight_words(C, KH, KW);
         char* base = static_cast<char*>(d_p4);
         int64_t* d_rows = reinterpret_cast<int64_t*>(base + gemm_route_plane_bytes(N, C, H, W));
@@ -832,10 +836,18 @@ int conv_f4_expanded(int type, const float* d_x, const float* d_thr, const void*
         e = launch_mfma_gemm(true, type, d_af, d_wf, M, OH * OW, KN, Kw, C * KH * KW, prelu_alpha, d_y, st);
         return e == hipSuccess ? FTNN_OK : hip_fail(e, "matrix-core GEMM launch");
     }
-    if (d_x) e = launch_quantize_f4(act_ternary, d_x, d_thr, N, C, H, W, d_p4, st);   // else d_p4 is ready
-    if (e != hipSuccess) return hip_fail(e, "fp4 quantize launch");
     const ConvGeom cg = {H, W, cpack_of(C), OH, OW, KW, cpack_of(C) * KH * KW, H_pad, W_pad, H_stride, W_stride,
                          make_fastdiv((uint32_t)OW), make_fastdiv((uint32_t)cpack_of(C)), make_fastdiv((uint32_t)KW)};
+    // many tiles, fp32 input and result: workgroup tiles staged through LDS, gathered from the quantised input in the
+    // tile kernel's own layout
+    if (tiles) {
+        e = launch_quantize_f4_tiled(act_ternary, d_x, d_thr, N, C, H, W, W_stride, d_p4, st);
+        if (e != hipSuccess) return hip_fail(e, "fp4 quantize launch");
+        e = launch_conv_f4_tiles(type, d_p4, d_wf, cg, N, KN, C * KH * KW, prelu_alpha, d_y, st);
+        return e == hipSuccess ? FTNN_OK : hip_fail(e, "fp4 conv tile launch");
+    }
+    if (d_x) e = launch_quantize_f4(act_ternary, d_x, d_thr, N, C, H, W, d_p4, st);   // else d_p4 is ready
+    if (e != hipSuccess) return hip_fail(e, "fp4 quantize launch");
     e = launch_conv_f4(type, d_p4, d_wf, cg, N, KN, C * KH * KW, prelu_alpha, d_y, st, qo);
     return e == hipSuccess ? FTNN_OK : hip_fail(e, "fp4 conv launch");
 }
@@ -980,7 +992,7 @@ int64_t ftnn_conv_scratch_bytes(int type, int N, int C, int H, int W, int KN, in
     }
     // enough for either engine, so that one buffer serves ftnn_conv and ftnn_conv_engine
     // fp4: operand region, fragments of the weights and, on the dense path, the re-packed weight rows
-    int64_t f4 = conv_f4_operand_bytes(N, C, H, W, KH, KW, OH, OW, KN) +
+    int64_t f4 = conv_f4_operand_bytes(N, C, H, W, KH, KW, OH, OW, KN, W_stride) +
                  (mfma_fragment_bytes(true, KN, conv_f4_weight_words(C, KH, KW)) + 255) / 256 * 256;
     if (dense_f4_applies(C, KH, KW)) f4 += (int64_t)KN * conv_f4_weight_words(C, KH, KW) * (wt ? 16 : 8);
     return bytes > f4 ? bytes : f4;
@@ -1148,7 +1160,7 @@ int ftnn_conv_engine(int engine, int type, const float* d_x, const float* d_thr,
         if (64LL * Kw >= (1LL << 24))
             return fail(FTNN_EINVAL, "K too long for exact fp32 accumulation; use the vector-ALU engine");
         if (!fits_f4) return fail(FTNN_EINVAL, "more than 2^31-1 input pixel words: use the vector-ALU engine");
-        char* d_wf = static_cast<char*>(d_scratch) + conv_f4_operand_bytes(N, C, H, W, KH, KW, OH, OW, KN);
+        char* d_wf = static_cast<char*>(d_scratch) + conv_f4_operand_bytes(N, C, H, W, KH, KW, OH, OW, KN, W_stride);
         const int64_t* rows = d_qw;
         hipError_t e;
         if (dense_f4_applies(C, KH, KW)) {   // the weights take the same re-packing first

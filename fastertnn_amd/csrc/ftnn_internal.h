@@ -272,6 +272,16 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
                           int K_unpack, float alpha, float* d_y, hipStream_t st, const QuantOut& qo = QuantOut());
 
 
+// the same layer as workgroup tiles of 128 x 128 or 256 x 256 staged through LDS (the GEMM kernel with its activation
+// fragments gathered from T4, the quantised input in the layout of launch_quantize_f4_tiled): for layers with
+// conv_f4_tile_route() and an fp32 result
+int64_t quantize_f4_tiled_bytes(int N, int C, int H, int W, int W_stride);
+hipError_t launch_quantize_f4_tiled(bool ternary, const float* d_x, const float* d_thr, int N, int C, int H, int W,
+                                    int W_stride, void* d_t4, hipStream_t st);
+bool conv_f4_tile_route(int64_t M, int KN, int CP, int taps, int64_t t4_bytes, int W_pad, int W_stride);
+hipError_t launch_conv_f4_tiles(int type, const void* d_p4, const void* d_wf, const ConvGeom& cg, int N, int KN,
+                                int K_unpack, float alpha, float* d_y, hipStream_t st);
+
 // ---- ftnn_api.hip ----  (arguments already validated)
 // The fp4 layer with weights expanded beforehand (d_wf: launch_mfma_expand(true, ...) of the packed rows).
 // d_x != null: the input is quantised into d_p4 (N*H*W*C_pack*32 bytes) first; d_x == null: d_p4 already
@@ -286,7 +296,7 @@ int conv_valu(int type, const float* d_x, const float* d_thr, const int64_t* d_q
               void* d_scratch, float* d_y, hipStream_t st, const QuantOut& qo, bool weights_prepared);
 // bytes of the fp4 layer's operand region (d_p4 above) for this shape, rounded up to 256: P4, or for a
 // few-channel layer the nibble pixels and dense rows
-int64_t conv_f4_operand_bytes(int N, int C, int H, int W, int KH, int KW, int OH, int OW, int KN);
+int64_t conv_f4_operand_bytes(int N, int C, int H, int W, int KH, int KW, int OH, int OW, int KN, int W_stride);
 // words per row of the weights as the fp4 layer reads them (the dense re-packing shortens them)
 int conv_f4_weight_words(int C, int KH, int KW);
 

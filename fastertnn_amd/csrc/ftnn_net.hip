@@ -209,7 +209,7 @@ ftnn_net_t* ftnn_net_create_ex(int batch, int n_layers, const ftnn_layer_t* laye
         for (const NetPart& part : net->parts) {
             if (f4[i])
                 max_p4 = std::max(max_p4, conv_f4_operand_bytes(part.batch, L.C, L.H, L.W, L.KH, L.KW, net->OH[i],
-                                                                net->OW[i], L.KN));
+                                                                net->OW[i], L.KN, L.stride));
             else
                 max_scratch = std::max(max_scratch, ftnn_conv_scratch_bytes(L.type, part.batch, L.C, L.H, L.W, L.KN, L.KH,
                                                                             L.KW, L.pad, L.pad, L.stride, L.stride));

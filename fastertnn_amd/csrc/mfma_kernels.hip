@@ -37,17 +37,19 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 // Ring of NS LDS buffers, each holding KF fragments (K words for fp4) per row-block: one barrier per KF fragments.
-// A workgroup of 2 x 2 wavefronts computes (64 WT) x (64 WT) results, a wavefront WT x WT blocks of 32 x 32:
-// WT = 4 for problems with enough 256 x 256 tiles to fill the chip, WT = 2 (128 x 128) below that.
-template <int WT, int KF, int NS>
+// A workgroup of 2 x 2 wavefronts computes (64 WTP) x (64 WTQ) results, a wavefront WTP x WTQ blocks of 32 x 32:
+// 4 x 4 for problems with enough 256 x 256 tiles to fill the chip, 2 x 2 (128 x 128) below that, 4 x 2 (256 kernels x
+// 128 pixels) for conv layers on the tile kernel, whose kernel side is the cheaper one to stage.
+template <int WTP, int WTQ, int KF, int NS>
 struct Tile {
-    static constexpr int RB = 2 * WT;             // row-blocks per operand side
-    static constexpr int FR = 2 * RB * KF;        // fragments per step: (RB P + RB Q row-blocks) x KF
-    static constexpr int FW = FR / 4;             // fragments staged by one wavefront per step
-    static constexpr int NL = 2 * WT;             // LDS reads per wavefront and k fragment
-    static constexpr int DPI = FW / NL;           // fragments a wavefront stages per LDS read of the last fragment
+    static constexpr int RBP = 2 * WTP, RBQ = 2 * WTQ;   // row-blocks per operand side
+    static constexpr int FR = (RBP + RBQ) * KF;          // fragments per step: the P row-blocks' first, then the Q ones'
+    static constexpr int FW = FR / 4;                    // fragments staged by one wavefront per step
+    static constexpr int NL = WTP + WTQ;                 // LDS reads per wavefront and k fragment
+    static constexpr int NM = WTP * WTQ;                 // multiplies per wavefront and k fragment
+    static constexpr int DPI = FW / NL;                  // fragments a wavefront stages per LDS read of the last fragment
     static constexpr size_t lds_bytes = (size_t)NS * FR * 1024;
-    static_assert(FW % NL == 0 && (WT * WT) % NL == 0, "whole staged fragments and WT/2 multiplies per LDS read");
+    static_assert(FR % 4 == 0 && FW % NL == 0, "whole staged fragments per wavefront and per LDS read");
     static_assert(NS >= 2 && KF % 2 == 0, "register sets alternate per fragment");
 };
 
@@ -174,14 +176,14 @@ __device__ __forceinline__ void dma16(const uint4* gsrc, uint32_t lds_byte_addr)
 // (f <= 0) f *= alpha", mm_p2_final_tnn_avx2.c:204-208; form 1 "r >= 0 ? r : alpha * r", mm_p2_final_tbn_avx2.c:73), stored
 // row-major (SWAP = false, OHW == 1) or in NCHW order.  Accumulator e of block (a, b): P row = 32 * (prb + a) + 8 * (e / 4)
 // + 4 * (lane / 32) + e % 4, Q row = 32 * (qrb + b) + lane % 32.
-template <bool F4, bool SWAP, int WT>
-__device__ __forceinline__ void store_tile(const typename Acc<F4>::type (&acc)[WT][WT], float* __restrict__ Y, int M, int KN,
+template <bool F4, bool SWAP, int WTP, int WTQ>
+__device__ __forceinline__ void store_tile(const typename Acc<F4>::type (&acc)[WTP][WTQ], float* __restrict__ Y, int M, int KN,
                                            int OHW, int prb, int qrb, int lane, int bias, int form, float alpha) {
     const bool le_form = form == 0;
 #pragma unroll
-    for (int a = 0; a < WT; a++)
+    for (int a = 0; a < WTP; a++)
 #pragma unroll
-        for (int b = 0; b < WT; b++) {
+        for (int b = 0; b < WTQ; b++) {
             const int q = (qrb + b) * 32 + (lane & 31);
             const int pbase = (prb + a) * 32 + 4 * (lane >> 5);
             size_t qoff;
@@ -213,114 +215,219 @@ __device__ __forceinline__ void store_tile(const typename Acc<F4>::type (&acc)[W
 // The epilogue computes r = acc - bias, then PReLU in the reference's form for the type:
 // form 0 "f = r; if (f <= 0) f *= alpha" (mm_p2_final_tnn_avx2.c:204-208), form 1
 // "r >= 0 ? r : alpha * r" (mm_p2_final_tbn_avx2.c:73).
-template <bool F4, bool SWAP, int WT, int kKF, int kNS>
+// IMPL (fp4, SWAP): a conv layer with implicit im2row.  Qf is then not a fragment array but the layer's quantised input
+// in the form T4[n][C_pack][half][row][column % s][column / s][16 bytes] (k_quantize_f4 with TILED): the two wavefronts
+// that stage the Q side compute, per fragment, each lane's own source address -- lane (pixel, K half) of the fragment of
+// K word w = (kh KW + kw) C_pack + ic reads its 16 bytes at input pixel (oh s + kh - p, ow s + kw - p) of plane ic, or a
+// the fill piece behind the planes (16 bytes of zeros, or of +1 nibbles for binary activations: the reference's
+// fill, src/tnns/ternarize2row_avx2.c:748-755, src/tnns/binarize2row_avx2.c:151) where that pixel lies outside the image or w is a padding word -- and the LDS-direct load drops the 64
+// lanes contiguously into the ring exactly as it drops a stored fragment.  In T4 the 32 pixels of a fragment half are
+// consecutive 16-byte pieces within an output row whatever the stride (records of 32 bytes gathered at the stride
+// took the load unit four times as many requests: 50 against 32 us on a 1024-channel 28 x 28 stride-2 layer).  The im2row rows and their expansion are never written (for a 1024-channel 56 x 56 layer:
+// 116 + 231 MB less traffic and two launches less), and everything behind the ring is the GEMM kernel unchanged.
+template <bool F4, bool SWAP, int WTP, int WTQ, int kKF, int kNS, bool IMPL = false>
 __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, const uint4* __restrict__ Qf,
                                               float* __restrict__ Y, int M, int KN, int OHW, int KB,
-                                              int bias, int form, float alpha) {
+                                              int bias, int form, float alpha, ConvGeom cg = ConvGeom(),
+                                              FastDiv dOHW = FastDiv(), int Ws = 0, FastDiv dSW = FastDiv()) {
+    static_assert(!IMPL || (F4 && SWAP), "implicit im2row: fp4 layer with the pixels along the lanes");
     extern __shared__ uint4 lds[];   // kNS buffers of kFR KiB
     typedef typename Acc<F4>::type acc_t;
-    typedef Tile<WT, kKF, kNS> TL;
-    constexpr int RB = TL::RB, kFR = TL::FR, kFW = TL::FW, NL = TL::NL, DPI = TL::DPI;
+    typedef Tile<WTP, WTQ, kKF, kNS> TL;
+    constexpr int RBP = TL::RBP, RBQ = TL::RBQ, kFR = TL::FR, kFW = TL::FW, NL = TL::NL, NM = TL::NM, DPI = TL::DPI;
+    constexpr int kPF = RBP * kKF;   // fragments of the P side per step
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wy = wave >> 1, wx = wave & 1;
     const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN;
-    const int prb0 = blockIdx.x * RB, qrb0 = blockIdx.y * RB;
+    const int prb0 = blockIdx.x * RBP, qrb0 = blockIdx.y * RBQ;
     const int prbmax = (prow + 31) / 32 - 1, qrbmax = (qrow + 31) / 32 - 1;
-    acc_t acc[WT][WT];
+    acc_t acc[WTP][WTQ];
 #pragma unroll
-    for (int a = 0; a < WT; a++)
+    for (int a = 0; a < WTP; a++)
 #pragma unroll
-        for (int b = 0; b < WT; b++)
+        for (int b = 0; b < WTQ; b++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[a][b][e] = 0;
 
-    // fragment f of a step: side f / (RB*kKF) (0 = P, 1 = Q), row-block (f / kKF) % RB, k fragment
-    // f % kKF; row-blocks past the operand are clamped (their results are never stored)
+    // fragment f of a step: the P side's kPF fragments first (row-block f / kKF, k fragment f % kKF), then the Q
+    // side's; row-blocks past the operand are clamped (their results are never stored)
     const uint4* src[kFW];
 #pragma unroll
     for (int i = 0; i < kFW; i++) {
         const int f = wave * kFW + i;
-        const int side = f / (RB * kKF), rbi = (f / kKF) % RB, kbi = f % kKF;
-        const uint4* base = side == 0 ? Pf + ((size_t)min(prb0 + rbi, prbmax) * KB + kbi) * 64
-                                      : Qf + ((size_t)min(qrb0 + rbi, qrbmax) * KB + kbi) * 64;
+        const bool qside = f >= kPF;
+        const int g = qside ? f - kPF : f, rbi = g / kKF, kbi = g % kKF;
+        const uint4* base = !qside ? Pf + ((size_t)min(prb0 + rbi, prbmax) * KB + kbi) * 64
+                                   : Qf + ((size_t)min(qrb0 + rbi, qrbmax) * KB + kbi) * 64;
         src[i] = base + lane;
     }
+    // IMPL: the Q side's fragments are gathered.  They are the last RBQ * kKF fragments of a step, staged by wavefront
+    // 3 and, where the tile is not square, by the tail of wavefront 2; a wavefront's Q fragments cover whole row blocks
+    // of 32 pixels, at most QMAX of them, from row block qfirst on.  A wavefront issues one instruction every few
+    // cycles, so what the gather adds per fragment must stay a handful of instructions:
+    //   * a table behind the ring, one entry per K word w = (kh KW + kw) C_pack + ic, holds what does not depend on
+    //     the lane: the bit of the word's tap (0 for a padding word), and the word's part of the piece index (plane,
+    //     tap row, column class and slot offset);
+    //   * per row block a lane keeps the mask of the taps that fall inside the image for its pixel, and its pixel's
+    //     part of the piece index;
+    // a fragment's source is then one AND, one add, one select and the address.
+    static_assert(!IMPL || kKF == 2, "two table entries per read");
+    static_assert(!IMPL || (kPF % kKF == 0 && kFW % kKF == 0 && kPF >= 2 * kFW), "Q fragments in whole row blocks, on wavefronts 2 and 3 only");
+    constexpr int QMAX = kFW / kKF;
+    const bool gathers = IMPL && (wave + 1) * kFW > kPF;   // wave-uniform: this wavefront stages Q fragments
+    const int qfirst = max(0, wave * kFW - kPF) / kKF;
+    uint32_t tapmask[IMPL ? QMAX : 1], pbase[IMPL ? QMAX : 1];
+    const uint32_t row16 = (uint32_t)(cg.W_stride * Ws);          // pieces per input row
+    const uint32_t half16 = (uint32_t)cg.H * row16;               // per half plane
+    const uint32_t fill_piece = (uint32_t)(cg.CP * 2) * half16 * (uint32_t)((M - 1) / OHW + 1);   // right behind the planes
+    uint2* const wtab = reinterpret_cast<uint2*>(lds + (size_t)kNS * kFR * 64);
+    if constexpr (IMPL) {
+        for (int w = tid; w < KB; w += 256) {
+            const int tap = (int)fastdiv((uint32_t)w, cg.dCP), ic = w - tap * cg.CP;
+            const int kh = (int)fastdiv((uint32_t)tap, cg.dKW), kw = tap - kh * cg.KW;
+            // column ow s + d with d = kw - pad: class d mod s, slot ow + floor(d / s) (d made non-negative by a
+            // multiple of s first: the host keeps the padding below 4096 s)
+            const uint32_t dd = (uint32_t)(kw - cg.W_pad + 4096 * cg.W_stride);
+            const uint32_t dq = fastdiv(dd, dSW), cls = dd - dq * (uint32_t)cg.W_stride;
+            wtab[w] = make_uint2(w < cg.K ? 1u << tap : 0u,
+                                 (uint32_t)ic * 2u * half16 + (uint32_t)kh * row16 + cls * (uint32_t)Ws + dq - 4096u);
+        }
+#pragma unroll
+        for (int j = 0; j < QMAX; j++) {
+            const int rb = min(qfirst + j, RBQ - 1);
+            const uint32_t q = (uint32_t)min((qrb0 + rb) * 32 + (lane & 31), M - 1);
+            const uint32_t img = fastdiv(q, dOHW);
+            const uint32_t pix = q - img * (uint32_t)OHW;
+            const int oh = (int)fastdiv(pix, cg.dOW), ow = (int)pix - oh * cg.OW;
+            const int ih0 = oh * cg.H_stride - cg.H_pad, iw0 = ow * cg.W_stride - cg.W_pad;
+            // (image, plane 0, this lane's half, row ih0, class 0, slot ow): wraps for a negative ih0, and the
+            // word's part brings it back whenever the tap is inside
+            pbase[j] = (img * (uint32_t)cg.CP * 2u + (uint32_t)(lane >> 5)) * half16 + (uint32_t)ih0 * row16 + (uint32_t)ow;
+            uint32_t m = 0u;
+            for (int kh = 0, tap = 0; kh < cg.K / (cg.CP * cg.KW); kh++)
+                for (int kw = 0; kw < cg.KW; kw++, tap++)
+                    m |= ((unsigned)(ih0 + kh) < (unsigned)cg.H && (unsigned)(iw0 + kw) < (unsigned)cg.W ? 1u : 0u) << tap;
+            tapmask[j] = m;
+        }
+        __syncthreads();   // the table is complete before the first stage is issued
+    }
+    // the table entries of the kKF words of the stage about to be issued (stages are issued strictly in order), read
+    // from LDS one stage ahead of their use (the table has two entries to spare behind its last word)
+    int g_w = kKF;
+    uint4 wt = make_uint4(0u, 0u, 0u, 0u), wt_ahead = make_uint4(0u, 0u, 0u, 0u);
+    if constexpr (IMPL) {
+        if (gathers) wt_ahead = *reinterpret_cast<const uint4*>(wtab);
+    }
+    auto next_words = [&]() {
+        wt = wt_ahead;
+        wt_ahead = *reinterpret_cast<const uint4*>(wtab + min(g_w, KB));
+        g_w += kKF;
+    };
+    // the gathered source of fragment i of wavefront W (both compile-time): its row block's slot in tapmask / pbase is
+    // then a constant
+    auto gathered = [&](auto wtag, int i) -> const uint4* {
+        constexpr int W = decltype(wtag)::value;
+        constexpr int first = (W * kFW > kPF ? W * kFW - kPF : 0) / kKF;
+        const int j = (W * kFW + i - kPF) / kKF - first;
+        const uint32_t bit = (i % kKF) == 0 ? wt.x : wt.z, off = (i % kKF) == 0 ? wt.y : wt.w;
+        const uint32_t piece = pbase[j] + off;
+        return Qf + ((tapmask[j] & bit) != 0u ? piece : fill_piece);   // a select on the index: no branch
+    };
     const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)lds);
     const int nstep = KB / kKF;
-    auto stage = [&](int step) {
-        const uint32_t dst = lds0 + (uint32_t)(step % kNS) * (kFR * 1024) + wave * (kFW * 1024);
-#pragma unroll
-        for (int i = 0; i < kFW; i++) dma16(src[i] + (size_t)step * kKF * 64, dst + i * 1024);
-    };
-    uint4 fa[2][WT], fb[2][WT];
+    uint4 fa[2][WTP], fb[2][WTQ];
     // one LDS read of fragment k of buffer `buf` into register set `set`, in the order the MFMAs
-    // consume them: i = 0: fa0, 1..WT: fb0..fb(WT-1), then fa1..fa(WT-1)
+    // consume them: i = 0: fa0, 1..WTQ: fb0..fb(WTQ-1), then fa1..fa(WTP-1)
     auto ldone = [&](int buf, int k, int set, int i) {
         const uint4* L = lds + (size_t)buf * kFR * 64;
-        if (i == 0) fa[set][0] = L[((wy * WT + 0) * kKF + k) * 64 + lane];
-        else if (i <= WT) fb[set][i - 1] = L[((RB + wx * WT + (i - 1)) * kKF + k) * 64 + lane];
-        else fa[set][i - WT] = L[((wy * WT + (i - WT)) * kKF + k) * 64 + lane];
+        if (i == 0) fa[set][0] = L[((wy * WTP + 0) * kKF + k) * 64 + lane];
+        else if (i <= WTQ) fb[set][i - 1] = L[((RBP + wx * WTQ + (i - 1)) * kKF + k) * 64 + lane];
+        else fa[set][i - WTQ] = L[((wy * WTP + (i - WTQ)) * kKF + k) * 64 + lane];
     };
-    // the WT/2 multiplies that go with LDS read i
+    // the multiplies that go with LDS read i: the NM of a k fragment spread evenly over its NL reads (WT / 2 each on a
+    // square tile), in the order (a, b) = (m / WTQ, m % WTQ)
     auto mfma2 = [&](int set, int i) {
 #pragma unroll
-        for (int j = 0; j < WT / 2; j++) {
-            const int m = (WT / 2) * i + j;
-            mfma<F4>(acc[m / WT][m % WT], fa[set][m / WT], fb[set][m % WT]);
-        }
+        for (int m = i * NM / NL; m < (i + 1) * NM / NL; m++) mfma<F4>(acc[m / WTQ][m % WTQ], fa[set][m / WTQ], fb[set][m % WTQ]);
     };
 
-    // prologue: the first kNS stages in flight, wait for stage 0 only
+    // The pipeline, instantiated per role of the wavefront so that no fragment's source is chosen at run time: role 0
+    // stages stored fragments only (every wavefront without IMPL; wavefronts 0 and 1 with it), roles 2 and 3 are
+    // wavefronts 2 and 3 under IMPL, whose Q fragments are gathered.  Every role passes the same barriers.
+    auto pipeline = [&](auto role_tag) {
+        constexpr int ROLE = decltype(role_tag)::value;
+        // source of the wavefront's fragment i for K step `step` (gathered: of the stage next_words() was last called for)
+        auto source = [&](int i, int step) -> const uint4* {
+            if constexpr (ROLE != 0) {
+                if (ROLE * kFW + i >= kPF) return gathered(role_tag, i);
+            }
+            return src[i] + (size_t)step * kKF * 64;
+        };
+        auto stage = [&](int step) {
+            const uint32_t dst = lds0 + (uint32_t)(step % kNS) * (kFR * 1024) + wave * (kFW * 1024);
+            if constexpr (ROLE != 0) next_words();
 #pragma unroll
-    for (int p = 0; p < kNS; p++)
-        if (p < nstep) stage(p);
-    if (nstep >= kNS) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFW * (kNS - 1)) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+            for (int i = 0; i < kFW; i++) dma16(source(i, step), dst + i * 1024);
+        };
+        // prologue: the first kNS stages in flight, wait for stage 0 only
 #pragma unroll
-    for (int i = 0; i < NL; i++) ldone(0, 0, 0, i);
+        for (int p = 0; p < kNS; p++)
+            if (p < nstep) stage(p);
+        if (nstep >= kNS) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFW * (kNS - 1)) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NL; i++) ldone(0, 0, 0, i);
 
-    auto step_body = [&](int s, auto full_tag) {
-        constexpr bool FULL = decltype(full_tag)::value;   // FULL: s + kNS < nstep
+        auto step_body = [&](int s, auto full_tag) {
+            constexpr bool FULL = decltype(full_tag)::value;   // FULL: s + kNS < nstep
 #pragma unroll
-        for (int k = 0; k < kKF; k++) {
-            const int set = k & 1;
-            if (k + 1 < kKF) {
+            for (int k = 0; k < kKF; k++) {
+                const int set = k & 1;
+                if (k + 1 < kKF) {
 #pragma unroll
-                for (int i = 0; i < NL; i++) {
-                    ldone(s % kNS, k + 1, set ^ 1, i);
-                    mfma2(set, i);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            } else {
-                // Last fragment of the step: all of this step is in registers.  Stage s+1 must
-                // have landed (stages s+2 .. s+kNS-1 may still be in flight); after the barrier
-                // buffer s % kNS is free for stage s+kNS.
-                if (FULL || s + kNS - 1 < nstep) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFW * (kNS - 2)) : "memory");
-                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                __syncthreads();
-                const bool do_ld = FULL || s + 1 < nstep;
-                const uint32_t dst = lds0 + (uint32_t)(s % kNS) * (kFR * 1024) + wave * (kFW * 1024);
-#pragma unroll
-                for (int i = 0; i < NL; i++) {
-                    if (FULL) {
-#pragma unroll
-                        for (int j = 0; j < DPI; j++)
-                            dma16(src[i * DPI + j] + (size_t)(s + kNS) * kKF * 64, dst + (i * DPI + j) * 1024);
+                    for (int i = 0; i < NL; i++) {
+                        ldone(s % kNS, k + 1, set ^ 1, i);
+                        mfma2(set, i);
+                        __builtin_amdgcn_sched_barrier(0);
                     }
-                    if (do_ld) ldone((s + 1) % kNS, 0, set ^ 1, i);
-                    mfma2(set, i);
-                    __builtin_amdgcn_sched_barrier(0);
+                } else {
+                    // Last fragment of the step: all of this step is in registers.  Stage s+1 must
+                    // have landed (stages s+2 .. s+kNS-1 may still be in flight); after the barrier
+                    // buffer s % kNS is free for stage s+kNS.
+                    if (FULL || s + kNS - 1 < nstep) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFW * (kNS - 2)) : "memory");
+                    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    __syncthreads();
+                    const bool do_ld = FULL || s + 1 < nstep;
+                    const uint32_t dst = lds0 + (uint32_t)(s % kNS) * (kFR * 1024) + wave * (kFW * 1024);
+                    if constexpr (FULL && ROLE != 0) next_words();
+#pragma unroll
+                    for (int i = 0; i < NL; i++) {
+                        if (FULL) {
+#pragma unroll
+                            for (int j = 0; j < DPI; j++) dma16(source(i * DPI + j, s + kNS), dst + (i * DPI + j) * 1024);
+                        }
+                        if (do_ld) ldone((s + 1) % kNS, 0, set ^ 1, i);
+                        mfma2(set, i);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
             }
-        }
+        };
+        int s = 0;
+        for (; s + kNS < nstep; s++) step_body(s, std::true_type{});
+        for (; s < nstep; s++) step_body(s, std::false_type{});
     };
-    int s = 0;
-    for (; s + kNS < nstep; s++) step_body(s, std::true_type{});
-    for (; s < nstep; s++) step_body(s, std::false_type{});
+    if constexpr (IMPL) {
+        if (wave == 3) pipeline(std::integral_constant<int, 3>{});
+        else if (wave == 2) pipeline(std::integral_constant<int, 2>{});
+        else pipeline(std::integral_constant<int, 0>{});
+    } else {
+        pipeline(std::integral_constant<int, 0>{});
+    }
 
-    store_tile<F4, SWAP, WT>(acc, Y, M, KN, OHW, prb0 + wy * WT, qrb0 + wx * WT, lane, bias, form, alpha);
+    store_tile<F4, SWAP, WTP, WTQ>(acc, Y, M, KN, OHW, prb0 + wy * WTP, qrb0 + wx * WTQ, lane, bias, form, alpha);
 }
 
 // ------------------------------------------------- fp4 operands at two bits per lane, offset codes
@@ -1039,24 +1146,25 @@ inline int64_t mfma_small_tile_below() {
 template <bool F4, bool SWAP, int WT, int KF, int NS>
 hipError_t launch_gemm_tile(const uint4* Pf, const uint4* Qf, float* Y, int M, int KN, int OHW, int KB,
                             int bias, int form, float alpha, hipStream_t st) {
-    auto kern = k_mfma<F4, SWAP, WT, KF, NS>;
-    constexpr size_t lds_bytes = Tile<WT, KF, NS>::lds_bytes;
+    auto kern = k_mfma<F4, SWAP, WT, WT, KF, NS>;
+    constexpr size_t lds_bytes = Tile<WT, WT, KF, NS>::lds_bytes;
     // the opt-in to more than 64 KiB of dynamic LDS is per kernel; done once, thread-safe
     // The kernel counts its LDS-direct loads by hand (s_waitcnt vmcnt(N)); a scratch access would be one more
     // vector-memory operation inside those windows, so a build of it that spills is refused (once per variant).
     static const hipError_t configured = []() {
-        const void* kern = reinterpret_cast<const void*>(&k_mfma<F4, SWAP, WT, KF, NS>);
+        const void* kern = reinterpret_cast<const void*>(&k_mfma<F4, SWAP, WT, WT, KF, NS>);
         hipFuncAttributes attr;
         hipError_t e = hipFuncGetAttributes(&attr, kern);
         if (e == hipSuccess && attr.localSizeBytes != 0) e = hipErrorLaunchFailure;
         if (e != hipSuccess) return e;
-        return hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)Tile<WT, KF, NS>::lds_bytes);
+        return hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)Tile<WT, WT, KF, NS>::lds_bytes);
     }();
     if (configured != hipSuccess) return configured;
     const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN, edge = 64 * WT;
     dim3 grid((prow + edge - 1) / edge, (qrow + edge - 1) / edge);
     if (grid.y > 65535) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, st, Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, st, Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha, ConvGeom(), FastDiv(), 0,
+                       FastDiv());
     return hipGetLastError();
 }
 
@@ -1188,6 +1296,79 @@ hipError_t launch_mfma_gemm_packed4(int type, const void* d_ac, const void* d_bc
     const int form = type == kTNN ? 0 : 1;
     return OHW > 1 ? launch_gemm_p4<true>(Bc, Ac, d_y, (int)M, KN, OHW, Kw / 2, sB, sA, off, form, alpha, st)
                    : launch_gemm_p4<false>(Ac, Bc, d_y, (int)M, KN, OHW, Kw / 2, sA, sB, off, form, alpha, st);
+}
+
+namespace {
+constexpr int kMaxTileRouteWords = 2040;   // K words per row the tile kernel keeps a table entry for (16 KiB of LDS with the two spare ones)
+template <int WTP, int WTQ, int NS>
+hipError_t launch_conv_tiles_wt(const uint4* Wf, const uint4* P4, float* Y, int M, int KN, int OHW, int KB, int bias, int form,
+                                float alpha, const ConvGeom& cg, hipStream_t st) {
+    auto kern = k_mfma<true, true, WTP, WTQ, 2, NS, true>;
+    typedef Tile<WTP, WTQ, 2, NS> TL;
+    constexpr size_t kLdsMax = 160u << 10;   // LDS of a compute unit
+    const size_t lds_bytes = TL::lds_bytes + (size_t)(KB + 2) * 8;   // the ring, then the table of K words (+ 2 read ahead)
+    if (KB > kMaxTileRouteWords || lds_bytes > kLdsMax) return hipErrorInvalidValue;
+    // as launch_gemm_tile: hand-counted LDS-direct loads, so no scratch; the LDS opt-in is per kernel
+    static const hipError_t configured = []() {
+        const void* k = reinterpret_cast<const void*>(&k_mfma<true, true, WTP, WTQ, 2, NS, true>);
+        hipFuncAttributes attr;
+        hipError_t e = hipFuncGetAttributes(&attr, k);
+        if (e == hipSuccess && attr.localSizeBytes != 0) e = hipErrorLaunchFailure;
+        if (e != hipSuccess) return e;
+        return hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsMax);
+    }();
+    if (configured != hipSuccess) return configured;
+    dim3 grid((KN + 64 * WTP - 1) / (64 * WTP), (M + 64 * WTQ - 1) / (64 * WTQ));   // P = weights, Q = pixels
+    if (grid.y > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, st, Wf, P4, Y, M, KN, OHW, KB, bias, form, alpha, cg,
+                       make_fastdiv((uint32_t)OHW), (cg.W + cg.W_stride - 1) / cg.W_stride, make_fastdiv((uint32_t)cg.W_stride));
+    return hipGetLastError();
+}
+}  // namespace
+
+// A layer goes to the tile kernel with implicit im2row from 150 tiles of 128 x 128 on, if its rows have at least 16
+// words and it has at least 512 output pixels.  Measured on MI355X, the reference's batch-8 stride-2 layers, quantiser
+// included: 512 channels at 56 x 56 (196 tiles) 38.6 -> 28.6 us, 1024 channels at 56 x 56 (392 tiles) 77.6 -> 60.4 us
+// (80 us as quantise + im2row + expansion + GEMM); with 98 and 104 tiles (256 channels at 56 x 56, 1024 at 28 x 28) the
+// layer kernel is as fast or faster (17.7 against 18.7, 31.8 against 33.1 us).  FTNN_CONV_TILES_FROM = n: tuning aid;
+// it sets the tile count and drops the conditions on words and pixels.
+bool conv_f4_tile_route(int64_t M, int KN, int CP, int taps, int64_t t4_bytes, int W_pad, int W_stride) {
+    static const char* tune = getenv("FTNN_CONV_TILES_FROM");
+    static const int64_t from = tune ? atoll(tune) : 150;
+    const int64_t tiles = ((M + 127) / 128) * ((KN + 127) / 128);
+    const int64_t K = (int64_t)CP * taps;
+    // the kernel's limits: a tap mask of 32 bits per pixel, a table entry per K word, 32-bit piece indices into T4, and
+    // its way of keeping kw - pad non-negative
+    return tiles >= from && (tune || (K >= 16 && M >= 512)) && taps <= 32 && (K + 3) / 4 * 4 <= kMaxTileRouteWords && M <= 0x7fffff00LL &&
+           t4_bytes / 16 <= 0x7fffffffLL && W_pad < 4096 * (int64_t)W_stride;
+}
+
+// A large conv layer as workgroup tiles staged through LDS, the activation fragments gathered from T4
+// (launch_quantize_f4_tiled; k_mfma with IMPL): fp32 NCHW result only.  d_wf: the weights as fp4 fragments
+// (KB = round4(cg.K) words per row).
+hipError_t launch_conv_f4_tiles(int type, const void* d_p4, const void* d_wf, const ConvGeom& cg, int N, int KN, int K_unpack,
+                                float alpha, float* d_y, hipStream_t st) {
+    const int OHW = cg.OH * cg.OW;
+    const int64_t M = (int64_t)N * OHW;
+    const int KB = round4(cg.K);
+    if (!conv_f4_tile_route(std::max<int64_t>(M, 1 << 30), 1 << 20, cg.CP, cg.K / cg.CP, quantize_f4_tiled_bytes(N, cg.CP * 64, cg.H, cg.W, cg.W_stride), cg.W_pad,
+                            cg.W_stride) || M > 0x7fffff00LL)
+        return hipErrorInvalidValue;   // beyond the kernel's limits (the tile count aside)
+    // BNN: every lane that is no real (channel, tap) is +1 x +1 in both operands, padding words included
+    const int bias = type == kBNN ? 64 * KB - K_unpack : 0;
+    const int form = type == kTNN ? 0 : 1;
+    const uint4* Wf = static_cast<const uint4*>(d_wf);
+    const uint4* P4 = static_cast<const uint4*>(d_p4);
+    // tile shape (kernels x pixels): FTNN_CONV_TILE_SHAPE = 22 | 42 | 44 forces one (tuning aid)
+    static const int tune = getenv("FTNN_CONV_TILE_SHAPE") ? atoi(getenv("FTNN_CONV_TILE_SHAPE")) : 0;
+    // 256 x 256 tiles once they fill the chip; 256 kernels x 128 pixels where those fill most of it in one round (the
+    // 1024-channel 56 x 56 layer at batch 8: 196 workgroups, 60.4 against 63.8 us on 392 tiles of 128 x 128); else 128 x 128
+    const int64_t big = ((M + 255) / 256) * ((KN + 255) / 256), mid = ((M + 127) / 128) * ((KN + 255) / 256);
+    int shape = big >= mfma_small_tile_below() ? 44 : (mid >= 180 ? 42 : 22);
+    if (tune == 22 || tune == 42 || tune == 44) shape = tune;
+    if (shape == 44) return launch_conv_tiles_wt<4, 4, 4>(Wf, P4, d_y, (int)M, KN, OHW, KB, bias, form, alpha, cg, st);
+    if (shape == 42) return launch_conv_tiles_wt<4, 2, 4>(Wf, P4, d_y, (int)M, KN, OHW, KB, bias, form, alpha, cg, st);
+    return launch_conv_tiles_wt<2, 2, 4>(Wf, P4, d_y, (int)M, KN, OHW, KB, bias, form, alpha, cg, st);
 }
 
 hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const ConvGeom& cg, int N, int KN,

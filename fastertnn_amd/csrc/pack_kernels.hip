@@ -86,10 +86,15 @@ __global__ __launch_bounds__(256) void k_quantize_pixels(const float* __restrict
 // (cleared bits, src/tnns/binarize2row_avx2.c:151).  Same block shape and loads as
 // k_quantize_pixels; a thread's 8 channels are one dword, transposed through LDS so that a
 // pixel's 32 bytes leave contiguously.
-template <bool TERN>
+// TILED: the operand of the tile kernel with implicit im2row instead (k_mfma, IMPL): the two 16-byte halves of a record in
+// planes of their own, and the columns of an image row sorted by column % stride_w, T4[n][C_pack][half][row][column %
+// s][column / s][16 bytes] with ceil(W / s) slots per class: the 32 lanes of a fragment half -- consecutive output
+// pixels, i.e. input columns s apart -- then read consecutive 16-byte pieces within an output row, whatever the stride.
+template <bool TERN, bool TILED = false>
 __global__ __launch_bounds__(256) void k_quantize_f4(const float* __restrict__ x,
                                                      const float* __restrict__ thr, int C, int HW,
-                                                     int CP, uint32_t* __restrict__ P4) {
+                                                     int CP, uint32_t* __restrict__ P4, int W = 0, int SW = 1, int Ws = 0,
+                                                     FastDiv dW = FastDiv(), FastDiv dSW = FastDiv()) {
     __shared__ uint32_t s_dw[32 * 9];
     const int px = threadIdx.x & 31, oct = threadIdx.x >> 5;
     const int p = blockIdx.x * 32 + px;
@@ -120,9 +125,31 @@ __global__ __launch_bounds__(256) void k_quantize_f4(const float* __restrict__ x
     }
     s_dw[px * 9 + oct] = dw;
     __syncthreads();
-    const int wp = threadIdx.x >> 3, wo = threadIdx.x & 7;
-    const int q = blockIdx.x * 32 + wp;
-    if (q < HW) P4[(((size_t)n * CP + ic) * HW + q) * 8 + wo] = s_dw[wp * 9 + wo];
+    if constexpr (TILED) {
+        // thread (pixel, half) stores the half record's 16 bytes
+        if (threadIdx.x < 64) {
+            const int wp = threadIdx.x & 31, half = threadIdx.x >> 5;
+            const int q = blockIdx.x * 32 + wp;
+            if (q < HW) {
+                const uint32_t ih = fastdiv((uint32_t)q, dW), iw = (uint32_t)q - ih * (uint32_t)W;
+                const uint32_t cls_q = fastdiv(iw, dSW), cls = iw - cls_q * (uint32_t)SW;
+                const int H = HW / W;
+                const size_t piece = ((((size_t)n * CP + ic) * 2 + half) * H + ih) * ((size_t)SW * Ws) + (size_t)cls * Ws + cls_q;
+                const uint32_t* d = s_dw + wp * 9 + half * 4;
+                reinterpret_cast<uint4*>(P4)[piece] = make_uint4(d[0], d[1], d[2], d[3]);
+            }
+        }
+        // the fill piece right behind the planes: what a tap outside the image contributes (0, or +1 for binary inputs)
+        if (threadIdx.x == 64 && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0) {
+            const uint32_t f = TERN ? 0u : 0x22222222u;
+            const int H = HW / W;
+            reinterpret_cast<uint4*>(P4)[(size_t)gridDim.z * CP * 2 * H * ((size_t)SW * Ws)] = make_uint4(f, f, f, f);
+        }
+    } else {
+        const int wp = threadIdx.x >> 3, wo = threadIdx.x & 7;
+        const int q = blockIdx.x * 32 + wp;
+        if (q < HW) P4[(((size_t)n * CP + ic) * HW + q) * 8 + wo] = s_dw[wp * 9 + wo];
+    }
 }
 
 // One wavefront ballot per 64-bit word: rows of J consecutive floats.
@@ -613,8 +640,25 @@ hipError_t launch_quantize_f4(bool ternary, const float* d_x, const float* d_thr
     const int CP = cpack_of(C), HW = H * W;
     dim3 grid((HW + 31) / 32, CP, N);
     uint32_t* P4 = static_cast<uint32_t*>(d_p4);
-    if (ternary) hipLaunchKernelGGL((k_quantize_f4<true>), grid, dim3(256), 0, st, d_x, d_thr, C, HW, CP, P4);
-    else hipLaunchKernelGGL((k_quantize_f4<false>), grid, dim3(256), 0, st, d_x, d_thr, C, HW, CP, P4);
+    if (ternary) hipLaunchKernelGGL((k_quantize_f4<true>), grid, dim3(256), 0, st, d_x, d_thr, C, HW, CP, P4, 0, 1, 0, FastDiv(), FastDiv());
+    else hipLaunchKernelGGL((k_quantize_f4<false>), grid, dim3(256), 0, st, d_x, d_thr, C, HW, CP, P4, 0, 1, 0, FastDiv(), FastDiv());
+    return hipGetLastError();
+}
+
+// bytes of T4 (k_quantize_f4 with TILED) for this input and column stride
+int64_t quantize_f4_tiled_bytes(int N, int C, int H, int W, int W_stride) {
+    return (int64_t)N * cpack_of(C) * 2 * H * W_stride * ((W + W_stride - 1) / W_stride) * 16 + 16;   // + the fill piece
+}
+
+hipError_t launch_quantize_f4_tiled(bool ternary, const float* d_x, const float* d_thr, int N, int C, int H, int W,
+                                    int W_stride, void* d_t4, hipStream_t st) {
+    const int CP = cpack_of(C), HW = H * W, Ws = (W + W_stride - 1) / W_stride;
+    dim3 grid((HW + 31) / 32, CP, N);
+    uint32_t* T4 = static_cast<uint32_t*>(d_t4);
+    const FastDiv dW = make_fastdiv((uint32_t)W), dSW = make_fastdiv((uint32_t)W_stride);
+    // slots of a class past its last column (W % s != 0) are never read: the gather reads real columns only
+    if (ternary) hipLaunchKernelGGL((k_quantize_f4<true, true>), grid, dim3(256), 0, st, d_x, d_thr, C, HW, CP, T4, W, W_stride, Ws, dW, dSW);
+    else hipLaunchKernelGGL((k_quantize_f4<false, true>), grid, dim3(256), 0, st, d_x, d_thr, C, HW, CP, T4, W, W_stride, Ws, dW, dSW);
     return hipGetLastError();
 }
 
