@@ -14,10 +14,11 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hi
          "-Wall", "-Wno-unused-function"]
 
 
-# Kernels that issue loads through inline asm and count them by hand (s_waitcnt vmcnt(N)): a register of theirs
-# that the compiler keeps in scratch memory could be the target of a load in flight, and every scratch access is
-# itself a vector-memory operation that moves the count the waits rely on.  The build refuses scratch use in
-# them (the library checks the same at run time before the first launch).  Source -> name fragments.
+# The tile GEMM kernels issue their LDS-direct loads through inline asm and count them by hand (s_waitcnt vmcnt(N)):
+# every scratch access is itself a vector-memory operation that moves the count the waits rely on, so the build
+# refuses scratch use in them (the library checks the same at run time before the first launch).  The layer kernels
+# use ordinary loads that the compiler counts; scratch there would only be slow, and is refused as a performance guard.
+# Source -> name fragments.
 NO_SCRATCH = {"mfma_kernels.hip": ("k_conv_f4", "k_mfma")}   # "k_mfma" covers k_mfma_p4 as well
 
 

@@ -35,6 +35,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
 // Ring of NS LDS buffers, each holding KF fragments (K words for fp4) per row-block: one barrier per KF fragments.
 // A workgroup of 2 x 2 wavefronts computes (64 WTP) x (64 WTQ) results, a wavefront WTP x WTQ blocks of 32 x 32:
@@ -58,8 +59,8 @@ struct Tile {
 // A group is 4 words (256 lanes) of a packed row: 16 dwords (8 sign, 8 zero) for ternary
 // rows, 8 dwords for binary rows.  Rows past `rows` expand to zeros.
 template <bool F4, bool TERN>
-__global__ __launch_bounds__(256) void k_expand(const uint32_t* __restrict__ P, int rows, int G,
-                                                uint4* __restrict__ out) {
+__device__ __forceinline__ void expand_block(const uint32_t* __restrict__ P, int rows, int G, uint4* __restrict__ out, int rb,
+                                             int gy, uint32_t* stage) {
     // A workgroup expands kGPB adjacent groups of its 32 rows: 256 contiguous bytes of each ternary row (128 of a
     // binary one).  They are fetched row-wise, 16 bytes per thread with neighbouring threads on neighbouring bytes,
     // and turned through LDS into the (row, dword) order the expansion works in: fetched in that order directly,
@@ -68,8 +69,7 @@ __global__ __launch_bounds__(256) void k_expand(const uint32_t* __restrict__ P, 
     constexpr int DPG = TERN ? 16 : 8;        // dwords per group and row
     constexpr int RD = kGPB * DPG;            // dwords per row in the block: 64 / 32
     constexpr int RS = RD + 1;                // LDS row stride: odd, the 32 rows of a read hit 32 banks
-    __shared__ uint32_t stage[32 * RS];
-    const int rb = blockIdx.x, g0 = blockIdx.y * kGPB, t = threadIdx.x;
+    const int g0 = gy * kGPB, t = threadIdx.x;
     {
         constexpr int PPR = RD / 4;           // 16-byte pieces per row: 16 / 8
         const int gmax = min(kGPB, G - g0) * (DPG / 4);   // pieces of a row that exist
@@ -135,6 +135,22 @@ __global__ __launch_bounds__(256) void k_expand(const uint32_t* __restrict__ P, 
             }
         }
     }
+}
+
+template <bool F4, bool TERN>
+__global__ __launch_bounds__(256) void k_expand(const uint32_t* __restrict__ P, int rows, int G, uint4* __restrict__ out) {
+    __shared__ uint32_t stage[32 * 65];
+    expand_block<F4, TERN>(P, rows, G, out, blockIdx.x, blockIdx.y, stage);
+}
+
+// both operands of a GEMM in one launch (the same K): the first ceil(rows_a / 32) workgroup columns expand A, the others B
+template <bool F4, bool TA, bool TB>
+__global__ __launch_bounds__(256) void k_expand2(const uint32_t* __restrict__ Pa, int rows_a, uint4* __restrict__ out_a,
+                                                 const uint32_t* __restrict__ Pb, int rows_b, uint4* __restrict__ out_b, int G) {
+    __shared__ uint32_t stage[32 * 65];
+    const int rba = (rows_a + 31) / 32;
+    if ((int)blockIdx.x < rba) expand_block<F4, TA>(Pa, rows_a, G, out_a, blockIdx.x, blockIdx.y, stage);
+    else expand_block<F4, TB>(Pb, rows_b, G, out_b, (int)blockIdx.x - rba, blockIdx.y, stage);
 }
 
 // ----------------------------------------------------------------------- GEMM
@@ -463,15 +479,13 @@ __global__ void k_zero_i32(int* __restrict__ p, int n, int* __restrict__ q, int 
 // grid (row blocks, groups / 4), block 256: as k_expand<true, TERN>, writing the packed4 layout (Kw words per row) and
 // adding the lanes of its rows into sums (zeroed before the launch)
 template <bool TERN>
-__global__ __launch_bounds__(256) void k_pack4(const uint32_t* __restrict__ P, int rows, int G, uint2* __restrict__ out,
-                                               int* __restrict__ sums) {
+__device__ __forceinline__ void pack4_block(const uint32_t* __restrict__ P, int rows, int G, uint2* __restrict__ out,
+                                            int* __restrict__ sums, int rb, int gy, uint32_t* stage, int* rowsum) {
     constexpr int kGPB = 4;
     constexpr int DPG = TERN ? 16 : 8;        // dwords per group and row
     constexpr int RD = kGPB * DPG;            // dwords per row in the block
     constexpr int RS = RD + 1;                // LDS row stride: odd, the 32 rows of a read hit 32 banks
-    __shared__ uint32_t stage[32 * RS];
-    __shared__ int rowsum[32];
-    const int rb = blockIdx.x, g0 = blockIdx.y * kGPB, t = threadIdx.x;
+    const int g0 = gy * kGPB, t = threadIdx.x;
     if (t < 32) rowsum[t] = 0;
     {
         constexpr int PPR = RD / 4;           // 16-byte pieces per row
@@ -519,6 +533,26 @@ __global__ __launch_bounds__(256) void k_pack4(const uint32_t* __restrict__ P, i
     atomicAdd(&rowsum[r], lanesum);
     __syncthreads();
     if (t < 32 && rb * 32 + t < rows) atomicAdd(&sums[rb * 32 + t], rowsum[t]);
+}
+
+template <bool TERN>
+__global__ __launch_bounds__(256) void k_pack4(const uint32_t* __restrict__ P, int rows, int G, uint2* __restrict__ out,
+                                               int* __restrict__ sums) {
+    __shared__ uint32_t stage[32 * 65];
+    __shared__ int rowsum[32];
+    pack4_block<TERN>(P, rows, G, out, sums, blockIdx.x, blockIdx.y, stage, rowsum);
+}
+
+// both operands of a GEMM in one launch, as k_expand2
+template <bool TA, bool TB>
+__global__ __launch_bounds__(256) void k_pack4_2(const uint32_t* __restrict__ Pa, int rows_a, uint2* __restrict__ out_a,
+                                                 int* __restrict__ sums_a, const uint32_t* __restrict__ Pb, int rows_b,
+                                                 uint2* __restrict__ out_b, int* __restrict__ sums_b, int G) {
+    __shared__ uint32_t stage[32 * 65];
+    __shared__ int rowsum[32];
+    const int rba = (rows_a + 31) / 32;
+    if ((int)blockIdx.x < rba) pack4_block<TA>(Pa, rows_a, G, out_a, sums_a, blockIdx.x, blockIdx.y, stage, rowsum);
+    else pack4_block<TB>(Pb, rows_b, G, out_b, sums_b, (int)blockIdx.x - rba, blockIdx.y, stage, rowsum);
 }
 
 // (P0, P1) of one K word -> the lane's 16 bytes of nibbles
@@ -762,8 +796,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
         iw0[b] = ow * cg.W_stride - cg.W_pad;
         pb[b] = n * (uint32_t)(cg.CP * cg.H * cg.W);   // image n of P4[n][C_pack][pixel]
     }
-    // threshold of each pixel block's image for the hand-over, fetched now: behind the hand-counted loads
-    // below the compiler could only place this load where its value is used, at the very end
+    // threshold of each pixel block's image for the hand-over, fetched now, in front of the K loop's loads
     float qthr[2] = {0.0f, 0.0f};
     if constexpr (QMODE != 0) {
 #pragma unroll
@@ -785,32 +818,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
             for (int e = 0; e < 16; e++) acc[a][b][e] = 0.0f;
 
     const uint32_t fillv = ABIN ? 0x22222222u : 0u;
-    // All four loads of a step are unconditional (a tap outside the image reads pixel 0 of its
-    // image and is replaced by the padding value before use) and issued through inline asm, so
-    // that they leave when the code says so -- two steps ahead of the step being multiplied --
-    // and not where the compiler would sink them, next to their use.  The kernel counts them by
-    // hand: `arrive` waits until at most 8 loads (two steps) are outstanding and ties that wait to
-    // the registers of the step about to be used.
-    auto ld16 = [](v4i& dst, const uint4* src) {
-        asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(dst) : "v"(src) : "memory");
-    };
-    // buffer descriptors (base, 48-bit; stride 0; bytes; raw 32-bit data format) and this lane's fixed offsets
-    v4i rsrc_x = {0, 0, 0, 0}, rsrc_w = {0, 0, 0, 0};
+    // All four loads of a step are unconditional (a tap outside the image reads pixel 0 of its image and is replaced
+    // by the padding value before use) and are issued two steps ahead of the step being multiplied.  They are ordinary
+    // loads (plain, or buffer-load builtins), so the compiler owns the dependency between a load and the use of its
+    // registers and places every s_waitcnt vmcnt itself; what keeps a load where the code issues it -- and not next to
+    // its use, where the scheduler would sink it -- is the scheduling fence after each step's loads (fence_loads).
+    auto ld16 = [](v4i& dst, const uint4* src) { dst = *reinterpret_cast<const v4i*>(src); };
+    // buffer descriptors (base; stride 0; bytes; raw 32-bit data format) and this lane's fixed offsets
+    __amdgpu_buffer_rsrc_t brs_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(P4), 0, (int)p4_bytes, 0x00020000);
+    __amdgpu_buffer_rsrc_t brs_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(Wf), 0, (int)wf_bytes, 0x00020000);
     uint32_t wofs[2] = {0u, 0u}, xofs[2] = {0u, 0u};
     if constexpr (BUF) {
-        const uint64_t px = reinterpret_cast<uint64_t>(P4), pw = reinterpret_cast<uint64_t>(Wf);
-        rsrc_x = v4i{__builtin_amdgcn_readfirstlane((int)(uint32_t)px), __builtin_amdgcn_readfirstlane((int)((px >> 32) & 0xffffu)),
-                     __builtin_amdgcn_readfirstlane((int)p4_bytes), 0x00020000};
-        rsrc_w = v4i{__builtin_amdgcn_readfirstlane((int)(uint32_t)pw), __builtin_amdgcn_readfirstlane((int)((pw >> 32) & 0xffffu)),
-                     __builtin_amdgcn_readfirstlane((int)wf_bytes), 0x00020000};
 #pragma unroll
         for (int a = 0; a < 2; a++) wofs[a] = ((uint32_t)min(kn0 / 32 + a, rbmax) * (uint32_t)KB * 64u + (uint32_t)lane) * 16u;
 #pragma unroll
         for (int b = 0; b < 2; b++)
             xofs[b] = ((pb[b] + (uint32_t)(ih0[b] * cg.W + iw0[b])) * 2u + (uint32_t)h) * 16u;
     }
-    auto ldbuf = [](v4i& dst, uint32_t voff, const v4i& rsrc, uint32_t soff) {
-        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(dst) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+    auto ldbuf = [&](v4i& dst, uint32_t voff, uint32_t soff, bool weights) {
+        const v4u v = __builtin_amdgcn_raw_buffer_load_b128(weights ? brs_w : brs_x, (int)voff, (int)soff, 0);
+        dst = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
     };
     auto load = [&](int w, ConvFrag& f) {   // w is wave-uniform
         const int tap = (int)fastdiv((uint32_t)w, cg.dCP), ic = w - tap * cg.CP;
@@ -818,7 +845,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
         if constexpr (BUF) {
             const uint32_t wsoff = (uint32_t)__builtin_amdgcn_readfirstlane(w) * 1024u;
 #pragma unroll
-            for (int a = 0; a < 2; a++) ldbuf(f.w[a], wofs[a], rsrc_w, wsoff);
+            for (int a = 0; a < 2; a++) ldbuf(f.w[a], wofs[a], wsoff, true);
             // byte offset of the record = this lane's part (xofs, fixed) + the word's part (scalar); the sum wraps
             // to the right value whenever the tap lies inside the image
             const uint32_t tapoff = (uint32_t)__builtin_amdgcn_readfirstlane((ic * HWin + kh * cg.W + kw) * 32);
@@ -828,7 +855,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
                 const bool in = (unsigned)ih < (unsigned)cg.H && (unsigned)iw < (unsigned)cg.W;
                 // ternary activations: an offset beyond p4_bytes returns the zeros that padding is; binary ones pad
                 // with +1, read record 0 instead and take the select in compute()
-                ldbuf(f.x[b], in ? xofs[b] + tapoff : (ABIN ? 0u : 0xffffff00u), rsrc_x, 0u);
+                ldbuf(f.x[b], in ? xofs[b] + tapoff : (ABIN ? 0u : 0xffffff00u), 0u, false);
                 f.in[b] = ABIN ? in : true;
             }
         } else {
@@ -844,12 +871,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
             }
         }
     };
-    auto arrive = [](ConvFrag& f, auto outstanding) {
-        asm volatile("s_waitcnt vmcnt(%4)"
-                     : "+v"(f.w[0]), "+v"(f.w[1]), "+v"(f.x[0]), "+v"(f.x[1])
-                     : "n"(decltype(outstanding)::value)
-                     : "memory");
-    };
+    auto fence_loads = []() { __builtin_amdgcn_sched_barrier(0); };   // the loads issued so far stay in front of this point
     auto compute = [&](const ConvFrag& f) {
         v8i x[2], wv[2];
 #pragma unroll
@@ -873,7 +895,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
     // re-read it and are not multiplied (whole rounds of NB steps).
     const int K = cg.K;
     ConvFrag f[NB];
-    std::integral_constant<int, 4 * (NB - 1)> ahead;
     int w = ks;
 #pragma unroll
     for (int j = 0; j < NB - 1; j++) load(min(w + S * j, K - 1), f[j]);
@@ -881,13 +902,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S == 1 && 
 #pragma unroll
         for (int j = 0; j < NB; j++) {
             load(min(w + S * (j + NB - 1), K - 1), f[(j + NB - 1) % NB]);
-            arrive(f[j], ahead);
+            fence_loads();
             if (j == 0 || w + S * j < K) compute(f[j]);
         }
     }
-    // the loads still in flight target live registers: drain them before anything reuses those
-#pragma unroll
-    for (int j = 0; j < NB; j++) arrive(f[j], std::integral_constant<int, 0>{});
 
     // hand-over: whether every lane of a pixel block may take the compare-free form
     DirectQuant direct_q[2] = {{false, false}, {false, false}};
@@ -1006,7 +1024,7 @@ __global__ __launch_bounds__(256) void k_conv_f4_small(const uint4* __restrict__
     const int ih0 = oh * cg.H_stride - cg.H_pad, iw0 = ow * cg.W_stride - cg.W_pad;
     const uint32_t pb = img * (uint32_t)(cg.CP * cg.H * cg.W);   // image of P4[n][C_pack][pixel]
     float qthr = 0.0f;
-    if constexpr (QMODE != 0) qthr = qo.thr[img];   // fetched ahead of the hand-counted loads (see k_conv_f4)
+    if constexpr (QMODE != 0) qthr = qo.thr[img];   // fetched in front of the K loop's loads (see k_conv_f4)
     const int HWin = cg.H * cg.W;
     const int rbmax = (KN + 31) / 32 - 1;
     const uint4* wb = Wf + (size_t)min(kn0 / 32, rbmax) * KB * 64 + lane;
@@ -1020,32 +1038,27 @@ __global__ __launch_bounds__(256) void k_conv_f4_small(const uint4* __restrict__
         v4i w, x;
         bool in;
     };
-    auto ld16 = [](v4i& dst, const uint4* src) {
-        asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(dst) : "v"(src) : "memory");
-    };
-    v4i rsrc_x = {0, 0, 0, 0}, rsrc_w = {0, 0, 0, 0};
+    auto ld16 = [](v4i& dst, const uint4* src) { dst = *reinterpret_cast<const v4i*>(src); };   // loads as in k_conv_f4
+    __amdgpu_buffer_rsrc_t brs_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(P4), 0, (int)p4_bytes, 0x00020000);
+    __amdgpu_buffer_rsrc_t brs_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(Wf), 0, (int)wf_bytes, 0x00020000);
     uint32_t wofs = 0u, xofs = 0u;
     if constexpr (BUF) {
-        const uint64_t px = reinterpret_cast<uint64_t>(P4), pw = reinterpret_cast<uint64_t>(Wf);
-        rsrc_x = v4i{__builtin_amdgcn_readfirstlane((int)(uint32_t)px), __builtin_amdgcn_readfirstlane((int)((px >> 32) & 0xffffu)),
-                     __builtin_amdgcn_readfirstlane((int)p4_bytes), 0x00020000};
-        rsrc_w = v4i{__builtin_amdgcn_readfirstlane((int)(uint32_t)pw), __builtin_amdgcn_readfirstlane((int)((pw >> 32) & 0xffffu)),
-                     __builtin_amdgcn_readfirstlane((int)wf_bytes), 0x00020000};
         wofs = ((uint32_t)min(kn0 / 32, rbmax) * (uint32_t)KB * 64u + (uint32_t)lane) * 16u;
         xofs = ((pb + (uint32_t)(ih0 * cg.W + iw0)) * 2u + (uint32_t)h) * 16u;
     }
-    auto ldbuf = [](v4i& dst, uint32_t voff, const v4i& rsrc, uint32_t soff) {
-        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(dst) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+    auto ldbuf = [&](v4i& dst, uint32_t voff, uint32_t soff, bool weights) {
+        const v4u v = __builtin_amdgcn_raw_buffer_load_b128(weights ? brs_w : brs_x, (int)voff, (int)soff, 0);
+        dst = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
     };
     auto load = [&](int w, Frag& f) {   // w is wave-uniform
         const int tap = (int)fastdiv((uint32_t)w, cg.dCP), ic = w - tap * cg.CP;
         const int kh = (int)fastdiv((uint32_t)tap, cg.dKW), kw = tap - kh * cg.KW;
         const int ih = ih0 + kh, iw = iw0 + kw;
         if constexpr (BUF) {
-            ldbuf(f.w, wofs, rsrc_w, (uint32_t)__builtin_amdgcn_readfirstlane(w) * 1024u);
+            ldbuf(f.w, wofs, (uint32_t)__builtin_amdgcn_readfirstlane(w) * 1024u, true);
             const bool in = (unsigned)ih < (unsigned)cg.H && (unsigned)iw < (unsigned)cg.W;
             const uint32_t tapoff = (uint32_t)__builtin_amdgcn_readfirstlane((ic * HWin + kh * cg.W + kw) * 32);
-            ldbuf(f.x, in ? xofs + tapoff : (ABIN ? 0u : 0xffffff00u), rsrc_x, 0u);   // as in k_conv_f4
+            ldbuf(f.x, in ? xofs + tapoff : (ABIN ? 0u : 0xffffff00u), 0u, false);   // as in k_conv_f4
             f.in = ABIN ? in : true;
         } else {
             ld16(f.w, wb + (size_t)w * 64);
@@ -1054,9 +1067,7 @@ __global__ __launch_bounds__(256) void k_conv_f4_small(const uint4* __restrict__
             ld16(f.x, P4 + o);
         }
     };
-    auto arrive = [](Frag& f, auto outstanding) {
-        asm volatile("s_waitcnt vmcnt(%2)" : "+v"(f.w), "+v"(f.x) : "n"(decltype(outstanding)::value) : "memory");
-    };
+    auto fence_loads = []() { __builtin_amdgcn_sched_barrier(0); };
     auto compute = [&](const Frag& f) {
         v8i x, wv;
 #pragma unroll
@@ -1070,7 +1081,6 @@ __global__ __launch_bounds__(256) void k_conv_f4_small(const uint4* __restrict__
     // as in k_conv_f4: register sets rotate by name, loads past the last word re-read it and are not multiplied
     const int K = cg.K;
     Frag f[NB];
-    std::integral_constant<int, 2 * (NB - 1)> ahead;
     int w = ks;
 #pragma unroll
     for (int j = 0; j < NB - 1; j++) load(min(w + S * j, K - 1), f[j]);
@@ -1078,12 +1088,10 @@ __global__ __launch_bounds__(256) void k_conv_f4_small(const uint4* __restrict__
 #pragma unroll
         for (int j = 0; j < NB; j++) {
             load(min(w + S * (j + NB - 1), K - 1), f[(j + NB - 1) % NB]);
-            arrive(f[j], ahead);
+            fence_loads();
             if (j == 0 || w + S * j < K) compute(f[j]);
         }
     }
-#pragma unroll
-    for (int j = 0; j < NB; j++) arrive(f[j], std::integral_constant<int, 0>{});
 
     if (ks != 0) {
         float4* dst = red + (size_t)((ks - 1) * 4) * 64 + lane;
@@ -1399,21 +1407,12 @@ hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const Co
     const uint4* P4 = static_cast<const uint4*>(d_p4);
     const uint4* Wf = static_cast<const uint4*>(d_wf);
     const FastDiv dOHW = make_fastdiv((uint32_t)OHW);
-    // The kernels' hand-counted loads write registers behind the compiler's back; that is only
-    // sound while none of their registers live in scratch memory, which is checked once per variant.
     // operand sizes: the buffer-load variants announce them in their descriptors
     const int64_t p4_bytes = (int64_t)N * cg.CP * cg.H * cg.W * 32, wf_bytes = (int64_t)((KN + 31) / 32) * KB * 1024;
     static const bool no_buf = getenv("FTNN_CONV_NO_BUFFER_LOADS") != nullptr;   // tuning aid
     const bool buf = !no_buf && p4_bytes <= 0xf0000000LL && wf_bytes <= 0xf0000000LL;
     auto launch64 = [&](auto variant) -> hipError_t {
         constexpr auto kern = decltype(variant)::value;
-        static const hipError_t sound = []() {
-            hipFuncAttributes attr;
-            hipError_t e = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(kern));
-            if (e == hipSuccess && attr.localSizeBytes != 0) e = hipErrorLaunchFailure;
-            return e;
-        }();
-        if (sound != hipSuccess) return sound;
         hipLaunchKernelGGL(kern, grid, dim3(64 * wpb), 0, st, P4, Wf, d_y, (int)M, KN, OHW, KB, bias, alpha, dOHW, cg, qo,
                            (uint32_t)std::min<int64_t>(p4_bytes, 0xffffffffLL), (uint32_t)std::min<int64_t>(wf_bytes, 0xffffffffLL));
         return hipGetLastError();
@@ -1474,18 +1473,41 @@ hipError_t launch_mm_mfma(bool f4, int type, const int64_t* d_a, const int64_t* 
         const int na = (int)na64, nb = (int)nb64;   // one launch zeroes both operands' row sums
         hipLaunchKernelGGL(k_zero_i32, dim3((na + nb + 255) / 256), dim3(256), 0, st, packed4_sums(Ac, M, Kw), na,
                            packed4_sums(Bc, KN, Kw), nb);
-        hipError_t e = launch_pack4(a_tern, d_a, (int)M, Kw, Ac, false, st);
-        if (e != hipSuccess) return e;
-        e = launch_pack4(b_tern, d_b, KN, Kw, Bc, false, st);
+        // both operands packed by one launch
+        const dim3 grid((unsigned)(na / 32 + nb / 32), (unsigned)((Kw / 4 + 3) / 4));
+        if (grid.y > 65535) return hipErrorInvalidValue;
+        const uint32_t *Ra = reinterpret_cast<const uint32_t*>(d_a), *Rb = reinterpret_cast<const uint32_t*>(d_b);
+        uint2 *Oa = static_cast<uint2*>(Ac), *Ob = static_cast<uint2*>(Bc);
+        int *Sa = packed4_sums(Ac, M, Kw), *Sb = packed4_sums(Bc, KN, Kw);
+#define FTNN_PACK2(TA_, TB_) hipLaunchKernelGGL((k_pack4_2<TA_, TB_>), grid, dim3(256), 0, st, Ra, (int)M, Oa, Sa, Rb, KN, Ob, Sb, Kw / 4)
+        if (a_tern && b_tern) FTNN_PACK2(true, true);
+        else if (a_tern) FTNN_PACK2(true, false);
+        else if (b_tern) FTNN_PACK2(false, true);
+        else FTNN_PACK2(false, false);
+#undef FTNN_PACK2
+        hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         return launch_mfma_gemm_packed4(type, Ac, Bc, M, OHW, KN, Kw, K_unpack, alpha, d_y, st);
     }
     void* Af = d_scratch;
     void* Bf = static_cast<char*>(d_scratch) + mfma_fragment_bytes(f4, M, Kw);
-    hipError_t e = launch_mfma_expand(f4, a_tern, d_a, (int)M, Kw, Af, st);
-    if (e != hipSuccess) return e;
-    e = launch_mfma_expand(f4, b_tern, d_b, KN, Kw, Bf, st);
-    if (e != hipSuccess) return e;
+    {   // both operands expanded by one launch
+        const dim3 grid((unsigned)((M + 31) / 32 + (KN + 31) / 32), (unsigned)((Kw / 4 + 3) / 4));
+        if (grid.y > 65535) return hipErrorInvalidValue;
+        const uint32_t *Ra = reinterpret_cast<const uint32_t*>(d_a), *Rb = reinterpret_cast<const uint32_t*>(d_b);
+        uint4 *Oa = static_cast<uint4*>(Af), *Ob = static_cast<uint4*>(Bf);
+#define FTNN_EXP2(F4_, TA_, TB_) hipLaunchKernelGGL((k_expand2<F4_, TA_, TB_>), grid, dim3(256), 0, st, Ra, (int)M, Oa, Rb, KN, Ob, Kw / 4)
+#define FTNN_EXP2T(F4_)                          \
+    if (a_tern && b_tern) FTNN_EXP2(F4_, true, true);  \
+    else if (a_tern) FTNN_EXP2(F4_, true, false);      \
+    else if (b_tern) FTNN_EXP2(F4_, false, true);      \
+    else FTNN_EXP2(F4_, false, false)
+        if (f4) { FTNN_EXP2T(true); } else { FTNN_EXP2T(false); }
+#undef FTNN_EXP2T
+#undef FTNN_EXP2
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     return launch_mfma_gemm(f4, type, Af, Bf, M, OHW, KN, Kw, K_unpack, alpha, d_y, st);
 }
 

@@ -153,7 +153,7 @@ def test_build_refuses_scratch_in_hand_counted_kernels():
           "x.hip:1:1: remark: Function Name: _ZN4ftnn8k_expandEvv [-Rpass-analysis=kernel-resource-usage]\n"
           "x.hip:1:1: remark:     ScratchSize [bytes/lane]: 64 [-Rpass-analysis=kernel-resource-usage]\n")
     build.check_no_scratch("mfma_kernels.hip", ok)   # scratch in a kernel that counts nothing by hand is no error
-    for kernel in ("k_conv_f4", "k_mfma"):           # in either hand-counted kernel it is
+    for kernel in ("k_conv_f4", "k_mfma"):           # in either guarded kernel it is
         lines = ok.splitlines(True)
         at = next(i for i, l in enumerate(lines) if kernel in l)
         lines[at + 1] = lines[at + 1].replace("lane]: 0", "lane]: 60")
