@@ -3,9 +3,9 @@ rocprofv3 counter runs of bench.py (one counter per run) and the plain device co
 with --copy-calibration.  bench.py reads that file for `roofline.traffic`; it holds no literal of its own.
 
     cd /tmp && export TMPDIR=/tmp
-    rocprofv3 --pmc FETCH_SIZE -d <repo>/gpurun_out/pmc_fetch -o r -- python3 <repo>/bench.py --cpu-rows 0 --no-extra --steps 3 --warmup 1 --copy-calibration
-    rocprofv3 --pmc WRITE_SIZE -d <repo>/gpurun_out/pmc_write -o r -- python3 <repo>/bench.py --cpu-rows 0 --no-extra --steps 3 --warmup 1 --copy-calibration
-    python3 bench_probe/traffic_from_pmc.py gpurun_out/pmc_fetch gpurun_out/pmc_write 8192 8192 32768
+    rocprofv3 --pmc FETCH_SIZE -d <out>/pmc_fetch -o r -- python3 <repo>/bench.py --cpu-rows 0 --no-extra --steps 3 --warmup 1 --copy-calibration
+    rocprofv3 --pmc WRITE_SIZE -d <out>/pmc_write -o r -- python3 <repo>/bench.py --cpu-rows 0 --no-extra --steps 3 --warmup 1 --copy-calibration
+    python3 bench_probe/traffic_from_pmc.py <out>/pmc_fetch <out>/pmc_write 8192 8192 32768
 
 Both counters report KiB per dispatch.  The calibration copy moves 256 MiB each way; the factor between that and what
 a counter reads for it scales every other dispatch of the same run.

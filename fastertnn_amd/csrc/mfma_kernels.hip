@@ -1340,15 +1340,22 @@ hipError_t launch_conv_tiles_wt(const uint4* Wf, const uint4* P4, float* Y, int 
 // (80 us as quantise + im2row + expansion + GEMM); with 98 and 104 tiles (256 channels at 56 x 56, 1024 at 28 x 28) the
 // layer kernel is as fast or faster (17.7 against 18.7, 31.8 against 33.1 us).  FTNN_CONV_TILES_FROM = n: tuning aid;
 // it sets the tile count and drops the conditions on words and pixels.
+namespace {
+// the tile kernel's limits: a tap mask of 32 bits per pixel, a table entry per K word, 32-bit piece indices into T4,
+// pixel indices below 2^31 and its way of keeping kw - pad non-negative
+bool conv_tiles_within_limits(int64_t M, int CP, int taps, int64_t t4_bytes, int W_pad, int W_stride) {
+    const int64_t K = (int64_t)CP * taps;
+    return taps <= 32 && (K + 3) / 4 * 4 <= kMaxTileRouteWords && M <= 0x7fffff00LL && t4_bytes / 16 <= 0x7fffffffLL &&
+           W_pad < 4096 * (int64_t)W_stride;
+}
+}  // namespace
+
 bool conv_f4_tile_route(int64_t M, int KN, int CP, int taps, int64_t t4_bytes, int W_pad, int W_stride) {
     static const char* tune = getenv("FTNN_CONV_TILES_FROM");
     static const int64_t from = tune ? atoll(tune) : 150;
     const int64_t tiles = ((M + 127) / 128) * ((KN + 127) / 128);
     const int64_t K = (int64_t)CP * taps;
-    // the kernel's limits: a tap mask of 32 bits per pixel, a table entry per K word, 32-bit piece indices into T4, and
-    // its way of keeping kw - pad non-negative
-    return tiles >= from && (tune || (K >= 16 && M >= 512)) && taps <= 32 && (K + 3) / 4 * 4 <= kMaxTileRouteWords && M <= 0x7fffff00LL &&
-           t4_bytes / 16 <= 0x7fffffffLL && W_pad < 4096 * (int64_t)W_stride;
+    return tiles >= from && (tune || (K >= 16 && M >= 512)) && conv_tiles_within_limits(M, CP, taps, t4_bytes, W_pad, W_stride);
 }
 
 // A large conv layer as workgroup tiles staged through LDS, the activation fragments gathered from T4
@@ -1359,9 +1366,8 @@ hipError_t launch_conv_f4_tiles(int type, const void* d_p4, const void* d_wf, co
     const int OHW = cg.OH * cg.OW;
     const int64_t M = (int64_t)N * OHW;
     const int KB = round4(cg.K);
-    if (!conv_f4_tile_route(std::max<int64_t>(M, 1 << 30), 1 << 20, cg.CP, cg.K / cg.CP, quantize_f4_tiled_bytes(N, cg.CP * 64, cg.H, cg.W, cg.W_stride), cg.W_pad,
-                            cg.W_stride) || M > 0x7fffff00LL)
-        return hipErrorInvalidValue;   // beyond the kernel's limits (the tile count aside)
+    if (!conv_tiles_within_limits(M, cg.CP, cg.K / cg.CP, quantize_f4_tiled_bytes(N, cg.CP * 64, cg.H, cg.W, cg.W_stride), cg.W_pad, cg.W_stride))
+        return hipErrorInvalidValue;
     // BNN: every lane that is no real (channel, tap) is +1 x +1 in both operands, padding words included
     const int bias = type == kBNN ? 64 * KB - K_unpack : 0;
     const int form = type == kTNN ? 0 : 1;

@@ -285,7 +285,10 @@ __global__ __launch_bounds__(KS ? 64 * KS : 256) void k_mm(const uint32_t* __res
                     za0[a] = za1[a] = make_uint4(0, 0, 0, 0);
                 }
             }
-            if (MODE == kTBN) {  // per-row zero count, src/tnns/mm_p2_final_tbn_avx2.c:44-52
+            // per-row zero count, src/tnns/mm_p2_final_tbn_avx2.c:44-52.  It depends on the row alone and the four
+            // wavefronts of a workgroup hold the same rows: each counts every fourth group, the sums meet after the loop
+            // (under the K split a wavefront's groups are its own anyway)
+            if (MODE == kTBN && (KS || ((g0 + g) & 3) == wave)) {
 #pragma unroll
                 for (int a = 0; a < TM; a++) {
                     bcnt_acc(rowz[a], za0[a].x);
@@ -318,6 +321,20 @@ __global__ __launch_bounds__(KS ? 64 * KS : 256) void k_mm(const uint32_t* __res
         __syncthreads();
     }
 
+    if constexpr (MODE == kTBN && !KS) {
+        // the loop's last barrier has passed: the operand buffers are free for the four partial zero counts of each row
+        static_assert(4 * BM <= 2 * BM * LDW, "the partial zero counts fit the operand buffers");
+        uint32_t* red = &lds[0][0];
+#pragma unroll
+        for (int a = 0; a < TM; a++) red[wave * BM + lane + 64 * a] = rowz[a];
+        __syncthreads();
+#pragma unroll
+        for (int a = 0; a < TM; a++) {
+            rowz[a] = 0;
+#pragma unroll
+            for (int w = 0; w < 4; w++) rowz[a] += red[w * BM + lane + 64 * a];
+        }
+    }
     if constexpr (KS) {
         // the loop's last barrier has passed: the operand buffers are free for the partial counts [wavefront - 1][count][lane]
         uint32_t* red = &lds[0][0];

@@ -112,7 +112,7 @@ FTNN_API float *mm_bnn(int64_t *a, int64_t *b, int N, int OH, int OW, int KN, in
  * weights (N, C, H, W) = (kernels, channels, kernel height, kernel width) with one threshold per kernel.  Each
  * returns aligned_alloc(32, ...) memory that the caller free()s.  A driver that links the reference's own utils.o
  * keeps the reference's definitions (the executable's symbols come first); to take these instead, compile that one
- * file with the three names renamed (INTEGRATION.md shows the line). */
+ * file with the three names renamed on the compiler's command line (-Dbitpacking2=ref_bitpacking2 and so on). */
 FTNN_API int64_t *bitpacking2(float *x, int I, int J);
 FTNN_API int64_t *ternarize_opt_avx2(float *x, float *q_thresholds, int N, int C, int H, int W);
 FTNN_API int64_t *binarize_opt_avx2(float *x, float *q_thresholds, int N, int C, int H, int W);
