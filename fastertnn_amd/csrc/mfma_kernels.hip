@@ -219,7 +219,7 @@ __device__ __forceinline__ void store_tile(const typename Acc<F4>::type (&acc)[W
                 const bool scale = le_form ? (fr <= 0.0f) : (r < 0);
                 const float f = scale ? fr * alpha : fr;
                 const size_t o = SWAP ? qoff + (size_t)p * OHW : (size_t)p * KN + qoff;
-                if (qok && p < (SWAP ? KN : M)) Y[o] = f;
+                if (qok && p < (SWAP ? KN : M)) __builtin_nontemporal_store(f, &Y[o]);
             }
         }
 }
@@ -599,7 +599,7 @@ __device__ __forceinline__ void store_tile_offset(const Acc<true>::type (&acc)[W
                 const bool scale = le_form ? (fr <= 0.0f) : (r < 0);
                 const float f = scale ? fr * alpha : fr;
                 const size_t o = SWAP ? qoff + (size_t)p * OHW : (size_t)p * KN + qoff;
-                if (qok && p < prow) Y[o] = f;
+                if (qok && p < prow) __builtin_nontemporal_store(f, &Y[o]);
             }
         }
     }
