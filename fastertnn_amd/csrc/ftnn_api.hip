@@ -1030,16 +1030,15 @@ int ftnn_mm(int type, const int64_t* d_a, const int64_t* d_b, int N, int OH, int
     return e == hipSuccess ? FTNN_OK : hip_fail(e, "mm launch");
 }
 
-// Engine choice by shape, from measurements on MI355X: the matrix-core path works on 256 x 256
-// tiles and pays two expansion passes (about 25 us of fixed cost), the vector-ALU kernel runs near
-// 0.3 PMAC/s.  fp4 wins from about 1.2e10 lane-MACs on, provided there are enough tiles to spread
-// over the CUs; below that the vector-ALU kernel is faster.
+// Engine choice by shape, from measurements on MI355X (m x m x 8m, whole calls from packed rows, device time): the
+// matrix-core path pays one launch that expands both operands and works on tiles of 64 x 64, 128 x 128 or 256 x 256 by
+// tile count; the vector-ALU kernel is one launch near 0.3 PMAC/s.  m = 512 (1.1e9 lane-MACs): 12.0 us on the vector
+// ALU against 13.3 us on fp4; 576 (1.5e9): 13.9 against 13.0; 640 (2.1e9): 17.8 against 13.3; 768: 23.8 against 15.1;
+// other shapes with 1.6e9 - 1.9e9 lane-MACs are ties within 1 us either way, hence fp4 from 2e9 on.
 static int select_engine(int type, int64_t M, int KN, int Kw) {
     (void)type;
-    // measured on MI355X: from about 5 GMAC the two expansions and the matrix-core kernel (128 x 128 tiles
-    // while 256 x 256 ones would leave compute units idle) take less time than the vector-ALU kernel
     const double lane_macs = (double)M * KN * 64.0 * Kw;
-    if (lane_macs >= 5e9 && KN >= 128 && Kw <= kMaxF4GemmWords) return FTNN_ENGINE_MFMA_F4;
+    if (lane_macs >= 2e9 && KN >= 128 && Kw <= kMaxF4GemmWords) return FTNN_ENGINE_MFMA_F4;
     return FTNN_ENGINE_VALU;
 }
 

@@ -1151,25 +1151,25 @@ inline int64_t mfma_small_tile_below() {
     return v;
 }
 
-template <bool F4, bool SWAP, int WT, int KF, int NS>
+template <bool F4, bool SWAP, int WTP, int WTQ, int KF, int NS>
 hipError_t launch_gemm_tile(const uint4* Pf, const uint4* Qf, float* Y, int M, int KN, int OHW, int KB,
                             int bias, int form, float alpha, hipStream_t st) {
-    auto kern = k_mfma<F4, SWAP, WT, WT, KF, NS>;
-    constexpr size_t lds_bytes = Tile<WT, WT, KF, NS>::lds_bytes;
+    auto kern = k_mfma<F4, SWAP, WTP, WTQ, KF, NS>;
+    constexpr size_t lds_bytes = Tile<WTP, WTQ, KF, NS>::lds_bytes;
     // the opt-in to more than 64 KiB of dynamic LDS is per kernel; done once, thread-safe
     // The kernel counts its LDS-direct loads by hand (s_waitcnt vmcnt(N)); a scratch access would be one more
     // vector-memory operation inside those windows, so a build of it that spills is refused (once per variant).
     static const hipError_t configured = []() {
-        const void* kern = reinterpret_cast<const void*>(&k_mfma<F4, SWAP, WT, WT, KF, NS>);
+        const void* kern = reinterpret_cast<const void*>(&k_mfma<F4, SWAP, WTP, WTQ, KF, NS>);
         hipFuncAttributes attr;
         hipError_t e = hipFuncGetAttributes(&attr, kern);
         if (e == hipSuccess && attr.localSizeBytes != 0) e = hipErrorLaunchFailure;
         if (e != hipSuccess) return e;
-        return hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)Tile<WT, WT, KF, NS>::lds_bytes);
+        return hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)Tile<WTP, WTQ, KF, NS>::lds_bytes);
     }();
     if (configured != hipSuccess) return configured;
-    const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN, edge = 64 * WT;
-    dim3 grid((prow + edge - 1) / edge, (qrow + edge - 1) / edge);
+    const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN;
+    dim3 grid((prow + 64 * WTP - 1) / (64 * WTP), (qrow + 64 * WTQ - 1) / (64 * WTQ));
     if (grid.y > 65535) return hipErrorInvalidValue;
     hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, st, Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha, ConvGeom(), FastDiv(), 0,
                        FastDiv());
@@ -1185,8 +1185,15 @@ hipError_t launch_gemm(const uint4* Pf, const uint4* Qf, float* Y, int M, int KN
     bool small = big < mfma_small_tile_below();
     // two fragments per step and a ring of four: four fragments per step with a ring of two (the same LDS, half
     // the barriers) measured 0.87 against 0.76 ms on 8192 x 8192 x 32768 -- the ring then no longer covers the loads
-    return small ? launch_gemm_tile<F4, SWAP, 2, 2, 4>(Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha, st)
-                 : launch_gemm_tile<F4, SWAP, 4, 2, 4>(Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha, st);
+    // Fewer than 112 tiles of 128 x 128 leave most compute units idle: tiles of 64 x 64 then, four K words per step
+    // (1024 x 1024 x 8192 as a whole call: 25.7 -> 19.0 us, 768: 21.2 -> 15.7, 1280 (100 tiles): 29.6 -> 27.2; from 144
+    // tiles on the larger tile is faster, 33.6 against 39.6 us at 1536; tiles of 128 x 64 lose everywhere).
+    // FTNN_MFMA_TINY_BELOW = n moves the threshold (tuning aid).
+    static const int tiny_below = getenv("FTNN_MFMA_TINY_BELOW") ? atoi(getenv("FTNN_MFMA_TINY_BELOW")) : 112;
+    const int64_t mid = (((int64_t)M + 127) / 128) * ((KN + 127) / 128);
+    if (small && mid < tiny_below) return launch_gemm_tile<F4, SWAP, 1, 1, 4, 4>(Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha, st);
+    return small ? launch_gemm_tile<F4, SWAP, 2, 2, 2, 4>(Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha, st)
+                 : launch_gemm_tile<F4, SWAP, 4, 4, 2, 4>(Pf, Qf, Y, M, KN, OHW, KB, bias, form, alpha, st);
 }
 
 template <bool F4>
@@ -1334,12 +1341,13 @@ hipError_t launch_conv_tiles_wt(const uint4* Wf, const uint4* P4, float* Y, int 
 }
 }  // namespace
 
-// A layer goes to the tile kernel with implicit im2row from 150 tiles of 128 x 128 on, if its rows have at least 16
+// A layer goes to the tile kernel with implicit im2row from 90 tiles of 128 x 128 on, if its rows have at least 16
 // words and it has at least 512 output pixels.  Measured on MI355X, the reference's batch-8 stride-2 layers, quantiser
 // included: 512 channels at 56 x 56 (196 tiles) 38.6 -> 28.6 us, 1024 channels at 56 x 56 (392 tiles) 77.6 -> 60.4 us
 // (80 us as quantise + im2row + expansion + GEMM); with 98 and 104 tiles (256 channels at 56 x 56, 1024 at 28 x 28) the
-// layer kernel is as fast or faster (17.7 against 18.7, 31.8 against 33.1 us).  FTNN_CONV_TILES_FROM = n: tuning aid;
-// it sets the tile count and drops the conditions on words and pixels.
+// layer kernel is as fast or faster than tiles of 128 x 128 (17.7 against 18.7, 31.8 against 33.1 us) and tiles of
+// 64 x 64 are faster than both (16.5 and 28.4 us); with 52 tiles (512 channels at 28 x 28) a tie, below that the layer
+// kernels win.  FTNN_CONV_TILES_FROM = n: tuning aid; it sets the tile count and drops the conditions on words and pixels.
 namespace {
 // the tile kernel's limits: a tap mask of 32 bits per pixel, a table entry per K word, 32-bit piece indices into T4,
 // pixel indices below 2^31 and its way of keeping kw - pad non-negative
@@ -1352,7 +1360,7 @@ bool conv_tiles_within_limits(int64_t M, int CP, int taps, int64_t t4_bytes, int
 
 bool conv_f4_tile_route(int64_t M, int KN, int CP, int taps, int64_t t4_bytes, int W_pad, int W_stride) {
     static const char* tune = getenv("FTNN_CONV_TILES_FROM");
-    static const int64_t from = tune ? atoll(tune) : 150;
+    static const int64_t from = tune ? atoll(tune) : 90;
     const int64_t tiles = ((M + 127) / 128) * ((KN + 127) / 128);
     const int64_t K = (int64_t)CP * taps;
     return tiles >= from && (tune || (K >= 16 && M >= 512)) && conv_tiles_within_limits(M, CP, taps, t4_bytes, W_pad, W_stride);
@@ -1373,15 +1381,18 @@ hipError_t launch_conv_f4_tiles(int type, const void* d_p4, const void* d_wf, co
     const int form = type == kTNN ? 0 : 1;
     const uint4* Wf = static_cast<const uint4*>(d_wf);
     const uint4* P4 = static_cast<const uint4*>(d_p4);
-    // tile shape (kernels x pixels): FTNN_CONV_TILE_SHAPE = 22 | 42 | 44 forces one (tuning aid)
+    // tile shape (kernels x pixels): FTNN_CONV_TILE_SHAPE = 11 | 22 | 42 | 44 forces one (tuning aid)
     static const int tune = getenv("FTNN_CONV_TILE_SHAPE") ? atoi(getenv("FTNN_CONV_TILE_SHAPE")) : 0;
     // 256 x 256 tiles once they fill the chip; 256 kernels x 128 pixels where those fill most of it in one round (the
-    // 1024-channel 56 x 56 layer at batch 8: 196 workgroups, 60.4 against 63.8 us on 392 tiles of 128 x 128); else 128 x 128
+    // 1024-channel 56 x 56 layer at batch 8: 196 workgroups, 60.4 against 63.8 us on 392 tiles of 128 x 128); else
+    // 128 x 128, and 64 x 64 below 150 of those
     const int64_t big = ((M + 255) / 256) * ((KN + 255) / 256), mid = ((M + 127) / 128) * ((KN + 255) / 256);
-    int shape = big >= mfma_small_tile_below() ? 44 : (mid >= 180 ? 42 : 22);
-    if (tune == 22 || tune == 42 || tune == 44) shape = tune;
+    const int64_t sq = ((M + 127) / 128) * ((KN + 127) / 128);
+    int shape = big >= mfma_small_tile_below() ? 44 : (mid >= 180 ? 42 : (sq >= 150 ? 22 : 11));
+    if (tune == 11 || tune == 22 || tune == 42 || tune == 44) shape = tune;
     if (shape == 44) return launch_conv_tiles_wt<4, 4, 4>(Wf, P4, d_y, (int)M, KN, OHW, KB, bias, form, alpha, cg, st);
     if (shape == 42) return launch_conv_tiles_wt<4, 2, 4>(Wf, P4, d_y, (int)M, KN, OHW, KB, bias, form, alpha, cg, st);
+    if (shape == 11) return launch_conv_tiles_wt<1, 1, 4>(Wf, P4, d_y, (int)M, KN, OHW, KB, bias, form, alpha, cg, st);
     return launch_conv_tiles_wt<2, 2, 4>(Wf, P4, d_y, (int)M, KN, OHW, KB, bias, form, alpha, cg, st);
 }
 

@@ -46,9 +46,9 @@ print("child ok")
 """
 
 
-@pytest.mark.parametrize("tile", ["22", "42", "44"])
+@pytest.mark.parametrize("tile", ["11", "22", "42", "44"])
 def test_tile_route_forced_on_small_and_ragged_layers(tile):
-    """tiles of 128 kernels x 128 pixels, 256 x 128 and 256 x 256"""
+    """tiles of 64 kernels x 64 pixels, 128 x 128, 256 x 128 and 256 x 256"""
     env = dict(os.environ, FTNN_CONV_TILES_FROM="1", FTNN_CONV_TILE_SHAPE=tile)
     print("case conv tile route forced, tile shape", tile, flush=True)
     r = subprocess.run([sys.executable, "-c", _CHILD, ROOT], env=env, capture_output=True, text=True, timeout=280)
@@ -56,10 +56,12 @@ def test_tile_route_forced_on_small_and_ragged_layers(tile):
 
 
 @pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
-def test_layer_that_takes_the_tile_route_by_itself(hip, oracle, typ):
-    """128 channels, 28 x 28, batch 13, 256 kernels: 160 tiles of 128 x 128, rows of 18 words"""
+@pytest.mark.parametrize("batch", [13, 8], ids=["160_tiles_of_128x128", "98_tiles_on_64x64"])
+def test_layer_that_takes_the_tile_route_by_itself(hip, oracle, typ, batch):
+    """128 channels, 28 x 28, 256 kernels, rows of 18 words: at batch 13 160 tiles of 128 x 128, at batch 8 98 of them,
+    which run as tiles of 64 x 64"""
     import torch
-    shape, batch = (128, 28, 28, 256, 3, 3, 1, 1), 13
+    shape = (128, 28, 28, 256, 3, 3, 1, 1)
     assert hip.conv_scratch_bytes(typ, batch, 128, 28, 28, 256, 3, 3, 1, 1) > 0
     L = make_layer(typ, shape, batch, seed=9300 + typ)
     print("case", TYPE_NAMES[typ], shape, batch, flush=True)

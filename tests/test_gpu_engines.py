@@ -125,6 +125,27 @@ def test_matrix_core_engines_with_256x256_tiles(hip, oracle, typ, shape):
 
 
 @pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
+@pytest.mark.parametrize("shape", [(1500, 1, 1, 1480, 4), (3, 23, 23, 1500, 8)], ids=["row_major", "nchw"])
+def test_matrix_core_engines_with_128x128_tiles(hip, oracle, typ, shape):
+    """on plain fragments (the int8 engine, fp4 whole calls with few 256 x 256 tiles) the tile kernel works on
+    64 x 64 tiles below 112 tiles of 128 x 128, as in the small cases above, and on 128 x 128 tiles from there
+    up to 160 tiles of 256 x 256: these cases are of that middle kind"""
+    n, oh, ow, kn, kw = shape
+    m = n * oh * ow
+    assert ((m + 127) // 128) * ((kn + 127) // 128) >= 112 and ((m + 255) // 256) * ((kn + 255) // 256) < 160
+    rng = np.random.default_rng(91 + typ + kw)
+    at, wt = act_is_ternary(typ), weight_is_ternary(typ)
+    a = rng.integers(-2 ** 63, 2 ** 63, size=m * kw * (2 if at else 1), dtype=np.int64)
+    b = rng.integers(-2 ** 63, 2 ** 63, size=kn * kw * (2 if wt else 1), dtype=np.int64)
+    ku = 64 * kw - 7
+    want = oracle.mm(typ, a, b, n, oh, ow, kn, kw, -0.5, ku)
+    a_d, b_d = _dev(a), _dev(b)
+    for eng in (hip.ENGINE_MFMA_I8, hip.ENGINE_MFMA_F4):
+        got = hip.mm_engine(eng, typ, a_d, b_d, n, oh, ow, kn, kw, -0.5, ku).cpu().numpy()
+        assert got.tobytes() == want.tobytes(), "engine %d" % eng
+
+
+@pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
 def test_weights_kept_in_engine_form_serve_every_batch(hip, oracle, typ):
     """ftnn_expand_rows once for the weights, then ftnn_mm_expanded for activations of several sizes: few rows (128 x 128
     tiles), many rows (256 x 256 tiles), a conv-shaped result; the engine form of an operand must not depend on the
