@@ -489,31 +489,52 @@ class Probe:
         return None if r is None else {"ms": round(r[0], 4), "shader_mhz": round(r[1], 1)}
 
 
+_GRID_SYNC_CHILD = r"""
+import ctypes as C, json, sys
+import torch
+lib = C.CDLL(sys.argv[1])
+lib.probe_gridsync_run.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double)]
+out = {}
+buf = (C.c_double * 4)()
+st = torch.cuda.current_stream().cuda_stream
+for mode, key in ((2, "launch_boundary"), (0, "cooperative_groups_grid_sync"), (1, "counter_barrier_bounded_wait")):
+    best = None
+    for _ in range(5):
+        if lib.probe_gridsync_run(mode, 1, 18, st, buf) != 0:
+            out = {"failed": key}
+            break
+        if buf[3] != 1.0:
+            out = {"failed": key + ": data passed through the synchronisations is wrong"}
+            break
+        best = buf[1] if best is None else min(best, buf[1])
+    if "failed" in out:
+        break
+    out[key + "_us"] = round(best, 2)
+    out["workgroups"] = int(buf[2])
+print("GRIDSYNC " + json.dumps(out), flush=True)
+"""
+
+
 def grid_sync_cost(torch):
     """bench_probe/libprobe_gridsync.so: microseconds per grid-wide synchronisation inside one cooperative launch (the
     library's cooperative_groups grid sync, and a counter barrier with a bounded wait) against microseconds per launch
     boundary of plain launches, 18 synchronisations each (a 19-layer chain), one workgroup of 256 threads per compute
-    unit.  What decides whether a chain of small layers should be one resident kernel."""
-    import ctypes as C
+    unit.  What decides whether a chain of small layers should be one resident kernel.  Runs in a child process: a
+    process that has made a cooperative launch ends in a segmentation fault inside rocprofv3's exit handler when it is
+    traced, which must not be this one's end (the child has printed its figures by then)."""
+    import subprocess
     path = os.path.join(ROOT, "bench_probe", "libprobe_gridsync.so")
     if not os.path.exists(path):
         return {"skipped": "bench_probe/libprobe_gridsync.so is not built"}
-    lib = C.CDLL(path)
-    lib.probe_gridsync_run.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double)]
-    out = {}
-    buf = (C.c_double * 4)()
-    st = torch.cuda.current_stream().cuda_stream
-    for mode, key in ((2, "launch_boundary"), (0, "cooperative_groups_grid_sync"), (1, "counter_barrier_bounded_wait")):
-        best = None
-        for _ in range(5):
-            if lib.probe_gridsync_run(mode, 1, 18, st, buf) != 0:
-                return {"failed": key}
-            if buf[3] != 1.0:
-                return {"failed": key + ": data passed through the synchronisations is wrong"}
-            best = buf[1] if best is None else min(best, buf[1])
-        out[key + "_us"] = round(best, 2)
-        out["workgroups"] = int(buf[2])
-    return out
+    try:
+        p = subprocess.run([sys.executable, "-c", _GRID_SYNC_CHILD, path], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                           text=True, timeout=120)
+    except subprocess.TimeoutExpired:
+        return {"failed": "timeout"}
+    for line in p.stdout.splitlines():
+        if line.startswith("GRIDSYNC "):
+            return json.loads(line[len("GRIDSYNC "):])
+    return {"failed": "child exit %d: %s" % (p.returncode, p.stderr[-300:])}
 
 
 def valu_reconciliation(torch, probe, run_valu, valu_ops, reps=12):
