@@ -241,12 +241,13 @@ __device__ __forceinline__ void store_tile(const typename Acc<F4>::type (&acc)[W
 // consecutive 16-byte pieces within an output row whatever the stride (records of 32 bytes gathered at the stride
 // took the load unit four times as many requests: 50 against 32 us on a 1024-channel 28 x 28 stride-2 layer).  The im2row rows and their expansion are never written (for a 1024-channel 56 x 56 layer:
 // 116 + 231 MB less traffic and two launches less), and everything behind the ring is the GEMM kernel unchanged.
-template <bool F4, bool SWAP, int WTP, int WTQ, int kKF, int kNS, bool IMPL = false>
+template <bool F4, bool SWAP, int WTP, int WTQ, int kKF, int kNS, bool IMPL = false, bool BAL = false>
 __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, const uint4* __restrict__ Qf,
                                               float* __restrict__ Y, int M, int KN, int OHW, int KB,
                                               int bias, int form, float alpha, ConvGeom cg = ConvGeom(),
                                               FastDiv dOHW = FastDiv(), int Ws = 0, FastDiv dSW = FastDiv()) {
     static_assert(!IMPL || (F4 && SWAP), "implicit im2row: fp4 layer with the pixels along the lanes");
+    static_assert(!BAL || IMPL, "the balanced assignment of fragments is for the gathering kernel");
     extern __shared__ uint4 lds[];   // kNS buffers of kFR KiB
     typedef typename Acc<F4>::type acc_t;
     typedef Tile<WTP, WTQ, kKF, kNS> TL;
@@ -268,10 +269,19 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
 
     // fragment f of a step: the P side's kPF fragments first (row-block f / kKF, k fragment f % kKF), then the Q
     // side's; row-blocks past the operand are clamped (their results are never stored)
+    // Which fragments a wavefront stages: in order (wavefront w the fragments w kFW .. w kFW + kFW - 1), or, BAL, a
+    // quarter of each side (PW fragments of the P side, then QW of the Q side), so that under IMPL every wavefront
+    // gathers the same number of fragments and none of them holds the others up at the step's barrier.
+    constexpr int PW = BAL ? kPF / 4 : 0, QW = BAL ? kFW - PW : 0;
+    static_assert(!BAL || (kPF % 4 == 0 && (QW % kKF == 0 || (QW == 1 && kKF == 2))), "a quarter of each side per wavefront");
+    auto frag_of = [&](int i) -> int {   // fragment number (its place in a stage of the ring) of the wavefront's slot i
+        if constexpr (BAL) return i < PW ? wave * PW + i : kPF + wave * QW + (i - PW);
+        else return wave * kFW + i;
+    };
     const uint4* src[kFW];
 #pragma unroll
     for (int i = 0; i < kFW; i++) {
-        const int f = wave * kFW + i;
+        const int f = frag_of(i);
         const bool qside = f >= kPF;
         const int g = qside ? f - kPF : f, rbi = g / kKF, kbi = g % kKF;
         const uint4* base = !qside ? Pf + ((size_t)min(prb0 + rbi, prbmax) * KB + kbi) * 64
@@ -289,10 +299,10 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
     //     part of the piece index;
     // a fragment's source is then one AND, one add, one select and the address.
     static_assert(!IMPL || kKF == 2, "two table entries per read");
-    static_assert(!IMPL || (kPF % kKF == 0 && kFW % kKF == 0 && kPF >= 2 * kFW), "Q fragments in whole row blocks, on wavefronts 2 and 3 only");
-    constexpr int QMAX = kFW / kKF;
-    const bool gathers = IMPL && (wave + 1) * kFW > kPF;   // wave-uniform: this wavefront stages Q fragments
-    const int qfirst = max(0, wave * kFW - kPF) / kKF;
+    static_assert(!IMPL || BAL || (kPF % kKF == 0 && kFW % kKF == 0 && kPF >= 2 * kFW), "Q fragments in whole row blocks, on wavefronts 2 and 3 only");
+    constexpr int QMAX = BAL ? (QW + kKF - 1) / kKF : kFW / kKF;
+    const bool gathers = IMPL && (BAL || (wave + 1) * kFW > kPF);   // wave-uniform: this wavefront stages Q fragments
+    const int qfirst = BAL ? (wave * QW) / kKF : max(0, wave * kFW - kPF) / kKF;
     uint32_t tapmask[IMPL ? QMAX : 1], pbase[IMPL ? QMAX : 1];
     const uint32_t row16 = (uint32_t)(cg.W_stride * Ws);          // pieces per input row
     const uint32_t half16 = (uint32_t)cg.H * row16;               // per half plane
@@ -344,9 +354,19 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
     // then a constant
     auto gathered = [&](auto wtag, int i) -> const uint4* {
         constexpr int W = decltype(wtag)::value;
-        constexpr int first = (W * kFW > kPF ? W * kFW - kPF : 0) / kKF;
-        const int j = (W * kFW + i - kPF) / kKF - first;
-        const uint32_t bit = (i % kKF) == 0 ? wt.x : wt.z, off = (i % kKF) == 0 ? wt.y : wt.w;
+        int j;
+        bool even;   // the fragment's K word within the stage
+        if constexpr (BAL) {
+            // slot i holds Q fragment w QW + (i - PW): with whole row blocks per wavefront both are compile-time; with one
+            // fragment per wavefront (QW == 1) the K word is the wavefront's parity
+            j = QW % kKF == 0 ? (i - PW) / kKF : 0;
+            even = QW % kKF == 0 ? ((i - PW) % kKF) == 0 : (wave & 1) == 0;
+        } else {
+            constexpr int first = (W * kFW > kPF ? W * kFW - kPF : 0) / kKF;
+            j = (W * kFW + i - kPF) / kKF - first;
+            even = (i % kKF) == 0;
+        }
+        const uint32_t bit = even ? wt.x : wt.z, off = even ? wt.y : wt.w;
         const uint32_t piece = pbase[j] + off;
         return Qf + ((tapmask[j] & bit) != 0u ? piece : fill_piece);   // a select on the index: no branch
     };
@@ -375,16 +395,18 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
         constexpr int ROLE = decltype(role_tag)::value;
         // source of the wavefront's fragment i for K step `step` (gathered: of the stage next_words() was last called for)
         auto source = [&](int i, int step) -> const uint4* {
-            if constexpr (ROLE != 0) {
+            if constexpr (BAL) {
+                if (i >= PW) return gathered(role_tag, i);
+            } else if constexpr (ROLE != 0) {
                 if (ROLE * kFW + i >= kPF) return gathered(role_tag, i);
             }
             return src[i] + (size_t)step * kKF * 64;
         };
         auto stage = [&](int step) {
-            const uint32_t dst = lds0 + (uint32_t)(step % kNS) * (kFR * 1024) + wave * (kFW * 1024);
+            const uint32_t dst = lds0 + (uint32_t)(step % kNS) * (kFR * 1024);
             if constexpr (ROLE != 0) next_words();
 #pragma unroll
-            for (int i = 0; i < kFW; i++) dma16(source(i, step), dst + i * 1024);
+            for (int i = 0; i < kFW; i++) dma16(source(i, step), dst + (uint32_t)frag_of(i) * 1024);
         };
         // prologue: the first kNS stages in flight, wait for stage 0 only
 #pragma unroll
@@ -416,13 +438,13 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
                     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                     __syncthreads();
                     const bool do_ld = FULL || s + 1 < nstep;
-                    const uint32_t dst = lds0 + (uint32_t)(s % kNS) * (kFR * 1024) + wave * (kFW * 1024);
+                    const uint32_t dst = lds0 + (uint32_t)(s % kNS) * (kFR * 1024);
                     if constexpr (FULL && ROLE != 0) next_words();
 #pragma unroll
                     for (int i = 0; i < NL; i++) {
                         if (FULL) {
 #pragma unroll
-                            for (int j = 0; j < DPI; j++) dma16(source(i * DPI + j, s + kNS), dst + (i * DPI + j) * 1024);
+                            for (int j = 0; j < DPI; j++) dma16(source(i * DPI + j, s + kNS), dst + (uint32_t)frag_of(i * DPI + j) * 1024);
                         }
                         if (do_ld) ldone((s + 1) % kNS, 0, set ^ 1, i);
                         mfma2(set, i);
@@ -435,7 +457,9 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
         for (; s + kNS < nstep; s++) step_body(s, std::true_type{});
         for (; s < nstep; s++) step_body(s, std::false_type{});
     };
-    if constexpr (IMPL) {
+    if constexpr (BAL) {
+        pipeline(std::integral_constant<int, 1>{});   // every wavefront stages and gathers alike
+    } else if constexpr (IMPL) {
         if (wave == 3) pipeline(std::integral_constant<int, 3>{});
         else if (wave == 2) pipeline(std::integral_constant<int, 2>{});
         else pipeline(std::integral_constant<int, 0>{});
@@ -1315,17 +1339,17 @@ hipError_t launch_mfma_gemm_packed4(int type, const void* d_ac, const void* d_bc
 
 namespace {
 constexpr int kMaxTileRouteWords = 2040;   // K words per row the tile kernel keeps a table entry for (16 KiB of LDS with the two spare ones)
-template <int WTP, int WTQ, int NS>
+template <int WTP, int WTQ, int NS, bool BAL>
 hipError_t launch_conv_tiles_wt(const uint4* Wf, const uint4* P4, float* Y, int M, int KN, int OHW, int KB, int bias, int form,
                                 float alpha, const ConvGeom& cg, hipStream_t st) {
-    auto kern = k_mfma<true, true, WTP, WTQ, 2, NS, true>;
+    auto kern = k_mfma<true, true, WTP, WTQ, 2, NS, true, BAL>;
     typedef Tile<WTP, WTQ, 2, NS> TL;
     constexpr size_t kLdsMax = 160u << 10;   // LDS of a compute unit
     const size_t lds_bytes = TL::lds_bytes + (size_t)(KB + 2) * 8;   // the ring, then the table of K words (+ 2 read ahead)
     if (KB > kMaxTileRouteWords || lds_bytes > kLdsMax) return hipErrorInvalidValue;
     // as launch_gemm_tile: hand-counted LDS-direct loads, so no scratch; the LDS opt-in is per kernel
     static const hipError_t configured = []() {
-        const void* k = reinterpret_cast<const void*>(&k_mfma<true, true, WTP, WTQ, 2, NS, true>);
+        const void* k = reinterpret_cast<const void*>(&k_mfma<true, true, WTP, WTQ, 2, NS, true, BAL>);
         hipFuncAttributes attr;
         hipError_t e = hipFuncGetAttributes(&attr, k);
         if (e == hipSuccess && attr.localSizeBytes != 0) e = hipErrorLaunchFailure;
@@ -1390,10 +1414,13 @@ hipError_t launch_conv_f4_tiles(int type, const void* d_p4, const void* d_wf, co
     const int64_t sq = ((M + 127) / 128) * ((KN + 127) / 128);
     int shape = big >= mfma_small_tile_below() ? 44 : (mid >= 180 ? 42 : (sq >= 150 ? 22 : 11));
     if (tune == 11 || tune == 22 || tune == 42 || tune == 44) shape = tune;
-    if (shape == 44) return launch_conv_tiles_wt<4, 4, 4>(Wf, P4, d_y, (int)M, KN, OHW, KB, bias, form, alpha, cg, st);
-    if (shape == 42) return launch_conv_tiles_wt<4, 2, 4>(Wf, P4, d_y, (int)M, KN, OHW, KB, bias, form, alpha, cg, st);
-    if (shape == 11) return launch_conv_tiles_wt<1, 1, 4>(Wf, P4, d_y, (int)M, KN, OHW, KB, bias, form, alpha, cg, st);
-    return launch_conv_tiles_wt<2, 2, 4>(Wf, P4, d_y, (int)M, KN, OHW, KB, bias, form, alpha, cg, st);
+    // 128 x 128 and 256 x 128 tiles: every wavefront gathers a quarter of the activation fragments (1024 channels at
+    // 56 x 56, batch 8: 60.2 -> 57.4 us; 512 channels: 27.3 -> 26.8); on 64 x 64 tiles the two gathering wavefronts of the
+    // plain order are faster (28.3 against 29.0 us), and 256 x 256 tiles have no registers to spare for four gatherers
+    if (shape == 44) return launch_conv_tiles_wt<4, 4, 4, false>(Wf, P4, d_y, (int)M, KN, OHW, KB, bias, form, alpha, cg, st);
+    if (shape == 42) return launch_conv_tiles_wt<4, 2, 4, true>(Wf, P4, d_y, (int)M, KN, OHW, KB, bias, form, alpha, cg, st);
+    if (shape == 11) return launch_conv_tiles_wt<1, 1, 4, false>(Wf, P4, d_y, (int)M, KN, OHW, KB, bias, form, alpha, cg, st);
+    return launch_conv_tiles_wt<2, 2, 4, true>(Wf, P4, d_y, (int)M, KN, OHW, KB, bias, form, alpha, cg, st);
 }
 
 hipError_t launch_conv_f4(int type, const void* d_p4, const void* d_wf, const ConvGeom& cg, int N, int KN,
