@@ -257,7 +257,20 @@ __global__ __launch_bounds__(256) void k_mfma(const uint4* __restrict__ Pf, cons
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wy = wave >> 1, wx = wave & 1;
     const int prow = SWAP ? KN : M, qrow = SWAP ? M : KN;
-    const int prb0 = blockIdx.x * RBP, qrb0 = blockIdx.y * RBQ;
+    // Tile of this workgroup.  Under IMPL the kernel tiles of one pixel tile read the same part of T4; workgroups are dealt
+    // to the eight XCDs round-robin by their linear number, so the tiles are renumbered to keep those on one XCD (its L2
+    // then fetches that part once, not once per kernel tile): XCD x takes the pixel tiles x, x + 8, ...; the pixel
+    // tiles beyond the last multiple of eight keep the plain order.
+    uint32_t bx = blockIdx.x, by = blockIdx.y;
+    if constexpr (IMPL) {
+        const uint32_t kt = gridDim.x, pt8 = gridDim.y / 8 * 8, lin = bx + kt * by;
+        if (lin < kt * pt8) {
+            const uint32_t xcd = lin & 7u, slot = lin >> 3;
+            by = xcd + 8u * (slot / kt);
+            bx = slot % kt;
+        }
+    }
+    const int prb0 = bx * RBP, qrb0 = by * RBQ;
     const int prbmax = (prow + 31) / 32 - 1, qrbmax = (qrow + 31) / 32 - 1;
     acc_t acc[WTP][WTQ];
 #pragma unroll
