@@ -166,15 +166,17 @@ def test_build_refuses_scratch_in_hand_counted_kernels():
 
 
 def test_benchmark_probe_is_built_outside_the_library():
-    """bench.py loads it for the measured vector-ALU issue rate; it is no part of the shipped package"""
+    """bench.py loads them for the measured vector-ALU issue rate and for the cost of a grid-wide synchronisation; they
+    are no part of the shipped package"""
     import ctypes
     import os
     from bench_probe import build as probe_build
     from fastertnn_amd import build
-    assert os.path.exists(build.LIB) and os.path.exists(probe_build.LIB)
+    assert os.path.exists(build.LIB) and os.path.exists(probe_build.LIB) and os.path.exists(probe_build.LIB_GRIDSYNC)
     dll = ctypes.CDLL(probe_build.LIB)
     for name in ("probe_valu_init", "probe_valu_run", "probe_clock_run", "probe_copy_run", "probe_mfma_run"):
         assert hasattr(dll, name)
+    assert hasattr(ctypes.CDLL(probe_build.LIB_GRIDSYNC), "probe_gridsync_run")
     assert not os.path.exists(os.path.join(os.path.dirname(build.LIB), "probe_valu"))
 
 
