@@ -5,7 +5,8 @@ Headline workload: the large compute-bound TNN GEMM (M = N = 8192, K = 32768,
 uniform ternary operands in Packing 2, PReLU(0.5) fused).  One "step" is one pass of
 the GEMM from two PACKED operands resident in HBM, as the reference's mm_tnn takes
 them: both are brought into the engine's operand form (ftnn_expand_rows) and
-multiplied (ftnn_mm_expanded) -- the launches of one ftnn_mm_engine call.  Where the
+multiplied (ftnn_mm_expanded) -- what one ftnn_mm_engine call does, as three calls so that
+the GEMM launch can be timed by itself (the one call is timed beside it).  Where the
 library's engine choice for the shape is the vector ALU the step is that one call.
 The step of a layer that keeps its weights in engine form is reported beside it
 (step_with_weights_kept_in_engine_form).  Prints ONE JSON line:
@@ -815,7 +816,8 @@ def main():
             lib.expand_rows(auto, a, m, kw, True, out=a_exp)
             lib.mm_expanded(auto, TNN, a_exp, b_exp, m, 1, 1, n, kw, alpha, out=y)
         step_desc = ("ftnn_expand_rows(A) + ftnn_expand_rows(B) + ftnn_mm_expanded: both operands from packed rows in "
-                     "every step, as mm_tnn takes them (the launches of one ftnn_mm_engine call)")
+                     "every step, as mm_tnn takes them (what one ftnn_mm_engine call does, as three calls so that the GEMM "
+                     "launch is timed by itself)")
 
     if args.copy_calibration:
         src = torch.empty(1 << 26, dtype=torch.float32, device="cuda").fill_(1.0)
