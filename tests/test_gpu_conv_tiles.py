@@ -72,3 +72,20 @@ def test_layer_that_takes_the_tile_route_by_itself(hip, oracle, typ, batch):
     assert got.cpu().numpy().tobytes() == want.tobytes()
     got = hip.host_conv(typ, L["x"], L["thr"], qw, L["kn"], 3, 3, 1, 1, 0.5)
     assert got.tobytes() == want.tobytes()
+
+
+@pytest.mark.parametrize("typ", ALL_TYPES, ids=lambda t: TYPE_NAMES[t])
+def test_single_layer_chain_takes_the_tile_route(hip, oracle, typ):
+    """a chain of one large layer (fp32 in, fp32 out) goes through the same route from ftnn_net_run: 160 tiles of
+    128 x 128 at batch 13, and at batch 50 the net's two half-batch chains with 225 tiles of 64 x 64 each"""
+    import torch
+    for shape, batch in (((128, 28, 28, 256, 3, 3, 1, 1), 13), ((256, 30, 30, 300, 3, 3, 1, 2), 50)):
+        L = make_layer(typ, shape, batch, seed=9500 + typ)
+        print("case", TYPE_NAMES[typ], shape, batch, flush=True)
+        qw = oracle.pack_weights(L["w"], L["wthr"], weight_is_ternary(typ))
+        thr = float(L["thr"][0])
+        want = oracle.conv(typ, L["x"], np.full(batch, thr, np.float32), qw, L["kn"], L["kh"], L["kw"], L["pad"], L["stride"], 0.5)
+        net = hip.Net(batch, [dict(type=typ, shape=shape, threshold=thr, alpha=0.5, qw=torch.from_numpy(qw).cuda())])
+        got = net.run(torch.from_numpy(L["x"]).cuda()).cpu().numpy()
+        net.close()
+        assert got.tobytes() == np.ascontiguousarray(want).tobytes()
