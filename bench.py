@@ -484,6 +484,20 @@ class Probe:
         return {"ms": round(r[0], 4), "tflops": round(r[1] / 1e12, 1), "frac_of_10100": round(r[1] / 10100e12, 4),
                 "shader_mhz": round(r[2], 1), "matrix_pipe_busy": round(r[3], 4)}
 
+    def lds_read_rate(self, torch, trips=20000):
+        """bytes per shader cycle and compute unit that wavefronts reading LDS with 16-byte reads reach (k_lds_read: four
+        wavefronts per workgroup, fragment layout), with one workgroup per compute unit -- how the 256 x 256 matrix-core
+        tiles run -- and with two"""
+        if self.lib is None or not hasattr(self.lib, "probe_lds_run"):
+            return None
+        res = {}
+        for wgs, key in ((1, "one_workgroup_per_cu"), (2, "two_workgroups_per_cu")):
+            out = (self.C.c_double * 2)()
+            if self.lib.probe_lds_run(wgs, int(trips), self.C.c_void_p(torch.cuda.current_stream().cuda_stream), out) != 0:
+                return None
+            res[key] = {"ms": round(out[0], 4), "bytes_per_cycle_and_cu": round(out[1], 1)}
+        return res
+
     def clock_after(self, torch, trips=16):
         """shader clock seen by a short, nearly idle kernel queued directly behind whatever ran last on the stream"""
         r = self._call(self.lib.probe_clock_run, trips, torch, 2)
@@ -983,6 +997,7 @@ def main():
             "reference_single_layers_b8": reference_single_layers(torch, lib),
             "reference_e2e_networks_b8": reference_networks(torch, lib, only=None if args.full else ("resnet18", "resnet152")),
             "grid_sync_against_launch_boundary": grid_sync_cost(torch),
+            "lds_read_rate_16_byte_reads": probe.lds_read_rate(torch) if probe.lib is not None else None,
         }
         if args.full:
             extra.update({

@@ -21,6 +21,11 @@
 //                     lanes are coded either as -1 / 0 / +1 (codes 0xA, 0x0, 0x2) or offset as 0 / 0.5 / 1 (codes
 //                     0, 1, 2, the form the GEMM's operands travel in): the clock differs between the two.
 //
+//   probe_lds_run     workgroups of four wavefronts, each wavefront reading its own KiBs of LDS with 16-byte reads
+//                     (ds_read_b128, lane l at byte 16 l: the layout of an MFMA operand fragment) and nothing else:
+//                     the bytes per cycle and compute unit that the matrix-core tile kernels' fragment reads can
+//                     reach with one workgroup per compute unit and with two.
+//
 // All are launched on the caller's stream and timed with HIP events recorded on that stream.
 #include <hip/hip_runtime.h>
 
@@ -142,6 +147,30 @@ double mean_mhz(int blocks) {
     return n ? sum / n : 0.0;
 }
 
+// Four wavefronts, each reading 8 fragments of 1 KiB per trip from its own 16 KiB of LDS; the addresses depend on the
+// trip and the values are kept alive, so that no read is hoisted out of the loop or dropped.
+__global__ __launch_bounds__(256) void k_lds_read(uint32_t* __restrict__ out, int trips, long long* __restrict__ cycles) {
+    __shared__ __attribute__((aligned(16))) uint32_t lds[16384];   // 64 KiB
+    for (int i = threadIdx.x; i < 16384; i += 256) lds[i] = (uint32_t)i;
+    __syncthreads();
+    typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t acc = 0u;
+    const long long t0 = clock64();
+    for (int it = 0; it < trips; it++) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t* base = lds + ((wave * 4096 + (it & 1) * 2048 + j * 256) & 16383);
+            const v4u v = *reinterpret_cast<const v4u*>(base + lane * 4);   // one ds_read_b128
+            asm volatile("" ::"v"(v));
+            acc += v.x;
+        }
+    }
+    const long long t1 = clock64();
+    out[blockIdx.x * 256 + threadIdx.x] = acc;
+    if (threadIdx.x == 0 && blockIdx.x == 0) *cycles = t1 - t0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -261,6 +290,27 @@ __attribute__((visibility("default"))) int probe_copy_run(const void* d_src, voi
     float ms = 0.0f;
     if (!ok(hipEventElapsedTime(&ms, g.e0, g.e1), "hipEventElapsedTime")) return 1;
     out[0] = ms;
+    return 0;
+}
+
+// `wgs_per_cu` (1 or 2) workgroups per compute unit, `trips` trips of 8 KiB per wavefront: out[0] = kernel ms, out[1] =
+// bytes read per shader cycle and compute unit (cycles counted by the first workgroup itself).
+__attribute__((visibility("default"))) int probe_lds_run(int wgs_per_cu, int trips, void* stream, double* out) {
+    if (probe_valu_init() != 0 || wgs_per_cu < 1 || wgs_per_cu > 2 || trips < 1) return 1;
+    static uint32_t* sink = nullptr;
+    static long long* cyc = nullptr;
+    if (!sink && (!ok(hipMalloc(&sink, (size_t)g.cus * 2 * 256 * 4), "hipMalloc") || !ok(hipMalloc(&cyc, 8), "hipMalloc"))) return 1;
+    hipStream_t st = (hipStream_t)stream;
+    if (!ok(hipEventRecord(g.e0, st), "hipEventRecord")) return 1;
+    hipLaunchKernelGGL(k_lds_read, dim3(g.cus * wgs_per_cu), dim3(256), 0, st, sink, trips, cyc);
+    long long c = 0;
+    if (!ok(hipGetLastError(), "launch") || !ok(hipEventRecord(g.e1, st), "hipEventRecord") ||
+        !ok(hipMemcpyAsync(&c, cyc, 8, hipMemcpyDeviceToHost, st), "copy") || !ok(hipStreamSynchronize(st), "sync"))
+        return 1;
+    float ms = 0.0f;
+    if (!ok(hipEventElapsedTime(&ms, g.e0, g.e1), "hipEventElapsedTime") || c <= 0) return 1;
+    out[0] = ms;
+    out[1] = (double)trips * 8 * 4 * 1024 * wgs_per_cu / (double)c;
     return 0;
 }
 

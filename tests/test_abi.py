@@ -174,7 +174,7 @@ def test_benchmark_probe_is_built_outside_the_library():
     from fastertnn_amd import build
     assert os.path.exists(build.LIB) and os.path.exists(probe_build.LIB) and os.path.exists(probe_build.LIB_GRIDSYNC)
     dll = ctypes.CDLL(probe_build.LIB)
-    for name in ("probe_valu_init", "probe_valu_run", "probe_clock_run", "probe_copy_run", "probe_mfma_run"):
+    for name in ("probe_valu_init", "probe_valu_run", "probe_clock_run", "probe_copy_run", "probe_mfma_run", "probe_lds_run"):
         assert hasattr(dll, name)
     assert hasattr(ctypes.CDLL(probe_build.LIB_GRIDSYNC), "probe_gridsync_run")
     assert not os.path.exists(os.path.join(os.path.dirname(build.LIB), "probe_valu"))
